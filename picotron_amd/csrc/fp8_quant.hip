@@ -1,0 +1,254 @@
+// Per-token-scaled FP8 E4M3 quantise / dequantise for gfx950 (HBM-bandwidth bound).
+//
+// Quantise, bf16 rows: one wavefront owns one row and keeps it in registers (each lane holds
+// 16-byte chunks lane, lane+64, ...), so HBM sees exactly one read of the row (2 B/elem) and one
+// write of the codes (1 B/elem) plus 4 B/row of scale.  amax is an integer max over the 15-bit
+// magnitudes (order-preserving for non-negative floats, and it carries NaN patterns to the top).
+//
+// The quotient float(x)/scale must be the IEEE-rounded one (the codes have to equal the ones a
+// plain fp32 division yields).  A full IEEE division per element would make the kernel ALU bound,
+// so each row computes r = RN(1/scale) once and every element uses the two-FMA correction
+//     q0 = x*r;  e = fma(-q0, scale, x);  q = fma(e, r, q0)
+// which is the correctly rounded quotient whenever r is the correctly rounded reciprocal and
+// nothing under/overflows (Markstein); rows whose scale is not finite take the plain division.
+#include "common.h"
+
+namespace {
+
+constexpr float kE4M3Max = 448.0f;
+constexpr uint32_t kAmaxFloorBf16 = 0x38D2u;  // bf16(1e-4)
+
+__device__ __forceinline__ float clamp448(float v) { return __builtin_amdgcn_fmed3f(v, -kE4M3Max, kE4M3Max); }
+
+// two fp32 -> two E4M3 codes placed in the low (hi_word = false) or high half of `old`
+template <bool HI>
+__device__ __forceinline__ uint32_t cvt2(float a, float b, uint32_t old) {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
+}
+
+struct RowScale {
+    float s;       // dequant multiplier as fp32
+    float r;       // RN(1/s)
+    bool finite;   // s is finite and non-NaN
+};
+
+__device__ __forceinline__ float quotient(float x, const RowScale& rs) {
+    float q0 = x * rs.r;
+    float e = __builtin_fmaf(-q0, rs.s, x);
+    return __builtin_copysignf(__builtin_fmaf(e, rs.r, q0), x);  // -0.0 / s must stay -0.0
+}
+
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void quant_bf16_wave_per_row(const u32x4_t* __restrict__ x, int64_t n_rows,
+                                                               int chunks_per_row, u32x2_t* __restrict__ q,
+                                                               float* __restrict__ scale) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;  // uniform per wave
+    const u32x4_t* xr = x + row * chunks_per_row;
+
+    u32x4_t v[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = c * 64 + lane;
+        v[c] = idx < chunks_per_row ? __builtin_nontemporal_load(xr + idx) : u32x4_t{0u, 0u, 0u, 0u};
+    }
+
+    typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+    u16x2 m2 = {0, 0};
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u16x2 a = __builtin_bit_cast(u16x2, w[i] & 0x7FFF7FFFu);
+            m2 = __builtin_elementwise_max(m2, a);
+        }
+    }
+    uint32_t amax_bits = m2.x > m2.y ? m2.x : m2.y;
+    amax_bits = wave_max(amax_bits);
+    const bool has_nan = amax_bits > 0x7F80u;
+    if (!has_nan && amax_bits < kAmaxFloorBf16) amax_bits = kAmaxFloorBf16;
+
+    RowScale rs;
+    rs.s = bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(amax_bits) / kE4M3Max));
+    rs.r = 1.0f / rs.s;
+    rs.finite = amax_bits < 0x7F80u;
+    if (lane == 0) scale[row] = rs.s;
+
+    u32x2_t* qr = q + row * chunks_per_row;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = c * 64 + lane;
+        const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+        if (rs.finite) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = clamp448(quotient(f[i], rs));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float t = f[i] / rs.s;
+                f[i] = (t != t) ? t : clamp448(t);
+            }
+        }
+        u32x2_t out;
+        out.x = cvt2<false>(f[0], f[1], 0u);
+        out.x = cvt2<true>(f[2], f[3], out.x);
+        out.y = cvt2<false>(f[4], f[5], 0u);
+        out.y = cvt2<true>(f[6], f[7], out.y);
+        if (idx < chunks_per_row) __builtin_nontemporal_store(out, qr + idx);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float load_as_f32(const T* p);
+template <>
+__device__ __forceinline__ float load_as_f32<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+
+// Any dtype / any hidden size: one 256-thread block per row, two passes over the row (the second
+// is served by L2).  T = float (fp32 rows) or uint16_t (bf16 bit patterns).
+template <typename T>
+__global__ __launch_bounds__(256) void quant_generic(const T* __restrict__ x, int64_t hidden, uint8_t* __restrict__ q,
+                                                     float* __restrict__ scale) {
+    __shared__ uint32_t part[4];
+    const int64_t row = blockIdx.x;
+    const T* xr = x + row * hidden;
+    uint32_t m = 0;  // fp32 magnitude bits (order preserving, NaN on top)
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        uint32_t b = __float_as_uint(load_as_f32<T>(xr + c)) & 0x7FFFFFFFu;
+        m = b > m ? b : m;
+    }
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = part[0];
+    for (int i = 1; i < 4; ++i) m = part[i] > m ? part[i] : m;
+    const bool has_nan = m > 0x7F800000u;
+    float amax = __uint_as_float(m);
+    float s;
+    if (sizeof(T) == 2) {
+        const float floor_v = bf16_bits_to_f32(kAmaxFloorBf16);
+        if (!has_nan && amax < floor_v) amax = floor_v;
+        s = bf16_bits_to_f32(f32_to_bf16_bits(amax / kE4M3Max));
+    } else {
+        if (!has_nan && amax < 1e-4f) amax = 1e-4f;
+        s = amax / kE4M3Max;
+    }
+    if (threadIdx.x == 0) scale[row] = s;
+    uint8_t* qr = q + row * hidden;
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        float t = load_as_f32<T>(xr + c) / s;
+        t = (t != t) ? t : clamp448(t);
+        qr[c] = (uint8_t)(cvt2<false>(t, t, 0u) & 0xFFu);
+    }
+}
+
+// ---- dequantise ------------------------------------------------------------------------------
+// bf16 out: 8 codes (one u32x2_t) per lane -> 8 bf16 (one u32x4_t).  float(code) * float(bf16(scale))
+// is exact in fp32 (4 x 8 significant bits), so one RNE to bf16 gives the reference's product.
+__global__ __launch_bounds__(256) void dequant_bf16_vec(const u32x2_t* __restrict__ q, const float* __restrict__ scale,
+                                                        int64_t n_rows, int chunks_per_row, u32x4_t* __restrict__ out) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const float s = bf16_bits_to_f32(f32_to_bf16_bits(scale[row]));
+    const u32x2_t* qr = q + row * chunks_per_row;
+    u32x4_t* orow = out + row * chunks_per_row;
+    for (int idx = lane; idx < chunks_per_row; idx += 64) {
+        const u32x2_t c = __builtin_nontemporal_load(qr + idx);
+        typedef __attribute__((ext_vector_type(2))) float f32x2;
+        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, false);
+        const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, true);
+        const f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, false);
+        const f32x2 e = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, true);
+        u32x4_t o;
+        o.x = pack_bf16x2(a.x * s, a.y * s);
+        o.y = pack_bf16x2(b.x * s, b.y * s);
+        o.z = pack_bf16x2(d.x * s, d.y * s);
+        o.w = pack_bf16x2(e.x * s, e.y * s);
+        __builtin_nontemporal_store(o, orow + idx);
+    }
+}
+
+template <bool BF16_OUT>
+__global__ __launch_bounds__(256) void dequant_generic(const uint8_t* __restrict__ q, const float* __restrict__ scale,
+                                                       int64_t hidden, void* __restrict__ out) {
+    const int64_t row = blockIdx.x;
+    const float s = BF16_OUT ? bf16_bits_to_f32(f32_to_bf16_bits(scale[row])) : scale[row];
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        const float v = __builtin_amdgcn_cvt_f32_fp8((int)q[row * hidden + c], 0) * s;
+        if (BF16_OUT)
+            ((uint16_t*)out)[row * hidden + c] = (uint16_t)f32_to_bf16_bits(v);
+        else
+            ((float*)out)[row * hidden + c] = v;
+    }
+}
+
+}  // namespace
+
+extern "C" int picomoe_fp8_quant(const void* x, int dtype, int64_t n_rows, int64_t hidden, uint8_t* q, float* scale,
+                                 void* stream) {
+    PICOMOE_CHECK_ARG(n_rows >= 0 && hidden > 0 && (dtype == PICOMOE_F32 || dtype == PICOMOE_BF16));
+    PICOMOE_CHECK_ARG(n_rows < (1ll << 31));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(x && q && scale);
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec_ok = dtype == PICOMOE_BF16 && hidden % 8 == 0 && hidden <= 8192 &&
+                        ((uintptr_t)x % 16 == 0) && ((uintptr_t)q % 8 == 0);
+    if (vec_ok) {
+        const int cpr = (int)(hidden / 8);
+        const int chunks = (cpr + 63) / 64;
+        const dim3 grid((unsigned)((n_rows + 3) / 4)), block(256);
+#define PICOMOE_LAUNCH_Q(C)                                                                                   \
+    hipLaunchKernelGGL(quant_bf16_wave_per_row<C>, grid, block, 0, st, (const u32x4_t*)x, n_rows, cpr, (u32x2_t*)q, \
+                       scale)
+        if (chunks <= 1) PICOMOE_LAUNCH_Q(1);
+        else if (chunks <= 2) PICOMOE_LAUNCH_Q(2);
+        else if (chunks <= 4) PICOMOE_LAUNCH_Q(4);
+        else if (chunks <= 8) PICOMOE_LAUNCH_Q(8);
+        else PICOMOE_LAUNCH_Q(16);
+#undef PICOMOE_LAUNCH_Q
+    } else if (dtype == PICOMOE_BF16) {
+        hipLaunchKernelGGL(quant_generic<uint16_t>, dim3((unsigned)n_rows), dim3(256), 0, st, (const uint16_t*)x, hidden,
+                           q, scale);
+    } else {
+        hipLaunchKernelGGL(quant_generic<float>, dim3((unsigned)n_rows), dim3(256), 0, st, (const float*)x, hidden, q,
+                           scale);
+    }
+    return picomoe_launch_status();
+}
+
+extern "C" int picomoe_fp8_dequant(const uint8_t* q, const float* scale, int64_t n_rows, int64_t hidden, void* out,
+                                   int dtype, void* stream) {
+    PICOMOE_CHECK_ARG(n_rows >= 0 && hidden > 0 && (dtype == PICOMOE_F32 || dtype == PICOMOE_BF16));
+    PICOMOE_CHECK_ARG(n_rows < (1ll << 31));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(q && scale && out);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == PICOMOE_BF16 && hidden % 8 == 0 && ((uintptr_t)q % 8 == 0) && ((uintptr_t)out % 16 == 0)) {
+        hipLaunchKernelGGL(dequant_bf16_vec, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, (const u32x2_t*)q, scale,
+                           n_rows, (int)(hidden / 8), (u32x4_t*)out);
+    } else if (dtype == PICOMOE_BF16) {
+        hipLaunchKernelGGL(dequant_generic<true>, dim3((unsigned)n_rows), dim3(256), 0, st, q, scale, hidden, out);
+    } else {
+        hipLaunchKernelGGL(dequant_generic<false>, dim3((unsigned)n_rows), dim3(256), 0, st, q, scale, hidden, out);
+    }
+    return picomoe_launch_status();
+}
+
+extern "C" int picomoe_abi_version(void) { return PICOMOE_ABI_VERSION; }
+
+extern "C" const char* picomoe_error_string(int code) {
+    if (code == PICOMOE_OK) return "ok";
+    if (code == PICOMOE_ERR_ARG) return "picomoe: unsupported shape, dtype, alignment or null pointer";
+    if (code >= PICOMOE_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(code - PICOMOE_ERR_HIP_BASE));
+    return "picomoe: unknown error code";
+}

@@ -1,0 +1,130 @@
+"""GPU parity of the FP8 E4M3 quantise / dequantise kernels against the CPU oracle: codes and
+scales bit-exact (called through the C ABI via picotron_amd.expert_parallel.ep_communications)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _c2_input(n, h, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, h, generator=g)
+    mask = torch.rand(n, h, generator=g) < 0.001
+    return torch.where(mask, 50 * torch.randn(n, h, generator=g), x)
+
+
+def _check(x_cpu, gpu):
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    q, s = C._per_token_quant_fp8(x_cpu.to(gpu))
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.float32
+    q_ref, s_ref = O.quant_fp8(x_cpu)
+    qc = q.view(torch.uint8).cpu()
+    bad = (qc != q_ref).nonzero()
+    assert bad.numel() == 0, f"{bad.shape[0]} code mismatches, first {bad[0].tolist()}: x={x_cpu[tuple(bad[0])].item()} got {qc[tuple(bad[0])].item()} want {q_ref[tuple(bad[0])].item()}"
+    assert torch.equal(s.cpu().view(torch.int32), s_ref.view(torch.int32))
+    d = C._dequant_fp8(q, s, x_cpu.dtype)
+    d_ref = O.dequant_fp8(q_ref, s_ref, x_cpu.dtype)
+    assert torch.equal(d.cpu().view(torch.int16 if x_cpu.dtype == torch.bfloat16 else torch.int32),
+                       d_ref.view(torch.int16 if x_cpu.dtype == torch.bfloat16 else torch.int32))
+    return q, s
+
+
+def test_quant_full_benchmark_shape_bit_exact(gpu):
+    """16384 x 4096 bf16, N(0,1) with 0.1% N(0,50) outliers: bytes and scales equal the reference cast."""
+    x = _c2_input(16384, 4096).bfloat16()
+    q, s = _check(x, gpu)
+    # size-independent properties on the same data
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    d = C._dequant_fp8(q, s, torch.bfloat16).float()
+    xf = x.to(gpu).float()
+    assert torch.all(d.abs().amax(-1) <= xf.abs().amax(-1).clamp_min(1e-4) * 1.005)
+    rel = ((d - xf).norm() / xf.norm()).item()
+    assert rel < 0.05, rel                       # the reference's own bound (tests/test_fp8_dispatch.py:85)
+    assert q.element_size() * q.shape[1] + s.element_size() == 4100
+
+
+@pytest.mark.parametrize("hidden", [8, 40, 256, 1000, 2048, 4104, 8192, 16384])
+def test_quant_row_widths_bf16(gpu, hidden):
+    x = _c2_input(67, hidden, seed=hidden).bfloat16()
+    _check(x, gpu)
+
+
+def test_quant_edge_rows_bf16(gpu):
+    x = _c2_input(16, 512, seed=5).bfloat16()
+    x[0] = 0                               # amax floor 1e-4
+    x[1] *= 1e-6                           # floor again, quotients below the smallest subnormal
+    x[2] *= 1e-3
+    x[3, 7] = 3.0e38                       # near bf16 max
+    x[4] = torch.tensor(1e-4).bfloat16()   # exactly the floor
+    x[5] = x[5].abs()
+    x[6] = -x[6].abs()
+    x[7, :] = 448.0
+    x[8, ::2] = 1.0
+    x[8, 1::2] = -1.0
+    _check(x, gpu)
+
+
+def test_quant_inf_row(gpu):
+    x = _c2_input(4, 256, seed=6).bfloat16()
+    x[1, 3] = float("inf")
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    q, s = C._per_token_quant_fp8(x.to(gpu))
+    q_ref, s_ref = O.quant_fp8(x)
+    finite_cols = torch.isfinite(x[1])
+    qc = q.view(torch.uint8).cpu()
+    assert torch.equal(qc[[0, 2, 3]], q_ref[[0, 2, 3]])
+    assert torch.equal(qc[1][finite_cols] & 0x7F, q_ref[1][finite_cols] & 0x7F)   # finite / inf = 0
+    assert (qc[1][~finite_cols] & 0x7F).tolist() == [0x7F]                         # inf / inf = NaN
+    assert torch.isinf(s.cpu()[1]) and torch.equal(s.cpu()[[0, 2, 3]], s_ref[[0, 2, 3]])
+
+
+def test_quant_adversarial_scales(gpu):
+    """Every bf16 value as an element, against scales whose mantissas stress the reciprocal trick
+    (all-ones, one, alternating) plus random ones."""
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    allv = allv[torch.isfinite(allv)]
+    rng = np.random.default_rng(0)
+    amax_bits = [0x3F80, 0x3FFF, 0x407F, 0x4000, 0x3FD5, 0x3FAA, 0x7F7F, 0x38D2, 0x3900, 0x43E0, 0x4460]
+    amax_bits += [int(b) for b in rng.integers(0x38D3, 0x7F7F, size=64)]
+    rows = []
+    for b in amax_bits:
+        amax = torch.tensor([b], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        row = torch.where(allv.abs() <= amax, allv, torch.zeros_like(allv))
+        row[0] = amax[0]
+        rows.append(row)
+    x = torch.stack(rows)[:, :65024]         # multiple of 8 columns -> generic path (hidden > 8192)
+    _check(x, gpu)
+    _check(x[:, :8192].contiguous(), gpu)    # vector path, row amax re-derived from the slice
+    _check(x[:, 30000:38192].contiguous(), gpu)
+
+
+@pytest.mark.parametrize("hidden", [16, 256, 1000])
+def test_quant_fp32_rows(gpu, hidden):
+    x = _c2_input(33, hidden, seed=hidden + 1)
+    x[0] = 0
+    _check(x, gpu)
+
+
+def test_cpu_tensor_is_refused():
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    with pytest.raises(_lib.PicomoeError):
+        C._per_token_quant_fp8(torch.randn(4, 8))
+
+
+def test_round_trip_autograd_is_straight_through(gpu):
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    x = _c2_input(32, 256, seed=9).bfloat16().to(gpu).requires_grad_(True)
+    y = C.fp8_round_trip(x)
+    g = torch.randn_like(y)
+    y.backward(g)
+    assert torch.equal(x.grad, g)
