@@ -46,6 +46,93 @@ int picomoe_fp8_quant(const void* x, int dtype, int64_t n_rows, int64_t hidden, 
 int picomoe_fp8_dequant(const uint8_t* q, const float* scale, int64_t n_rows, int64_t hidden, void* out, int dtype,
                         void* stream);
 
+/* ---- Router --------------------------------------------------------------------------------------
+ * Replaces EP/expert_parallel.py:175-184 (MoELayer._route after the gate Linear): probs =
+ * softmax_fp32(logits [n_tokens, num_experts]); picks = top_k of (probs + expert_bias) ordered by
+ * descending score, lower expert id first on equal scores; weights = probs at the picks, divided by
+ * their sum when norm_topk != 0 and top_k > 1, cast to dtype.  num_experts <= 1024, top_k <= 16.
+ * Optional outputs (NULL to skip): probs [n_tokens, num_experts] fp32; counts [num_experts] int32
+ * (picks per expert are ADDED with integer atomics: zero it first); colsum_partial
+ * [picomoe_route_partials(...), num_experts] fp32 partial column sums of probs (EP/expert_parallel.py:196-203). */
+int picomoe_route_partials(int64_t n_tokens, int num_experts);
+int picomoe_route_fwd(const void* logits, int dtype, int64_t n_tokens, int num_experts, int top_k,
+                      const float* expert_bias, int norm_topk, int64_t* topk_idx, void* topk_w, float* probs,
+                      int* counts, float* colsum_partial, void* stream);
+
+/* Backward of the above plus the aux-loss term (autograd of EP/expert_parallel.py:175-184 and :202-204):
+ * d_logits = softmax_bwd(d_probs) with d_probs gathering d_topk_w (through the renormalisation) and
+ * d_aux[0] * aux_coef * f_e / n_tokens, f_e = counts[e] * E / (top_k * n_tokens).  d_topk_w, d_aux, counts
+ * may be NULL. */
+int picomoe_route_bwd(const float* probs, const int64_t* topk_idx, const void* d_topk_w, int dtype, int64_t n_tokens,
+                      int num_experts, int top_k, int norm_topk, const float* d_aux, const int* counts, float aux_coef,
+                      void* d_logits, void* stream);
+
+/* Replaces EP/expert_parallel.py:199-212 (MoELayer._balance): aux_out[0] = aux_coef * sum_e f_e * mean_t probs[t,e]
+ * (skipped when aux_out is NULL) and expert_bias[e] += bias_rate * sign(mean(counts) - counts[e]) in place
+ * (skipped when expert_bias is NULL or bias_rate == 0). */
+int picomoe_balance(const int* counts, const float* colsum_partial, int n_partials, int64_t n_tokens, int num_experts,
+                    int top_k, float aux_coef, float bias_rate, float* aux_out, float* expert_bias, void* stream);
+
+/* ---- Permute / unpermute (the EP=1 form of dispatch / combine) ---------------------------------------
+ * Replaces EP/expert_parallel.py:30-35 and :335-339 (stable argsort by expert, its inverse, bincount) and
+ * EP/capacity_moe.py:44-57, :109-110 (_slot_assignment and the drop-mode keep mask).
+ * expert_idx [n_rows] int64.  Rows are ranked inside their expert in ascending row order (within[r]); with
+ * capacity > 0 only rows whose rank lies in [round_index*capacity, (round_index+1)*capacity) are kept (round 0
+ * alone is the drop mode; successive rounds are the static-memory dropless loop, EP/capacity_moe.py:108-110).
+ * Kept rows are laid out expert after expert:
+ * inv_order[r] = sorted position of row r, or -1 when dropped; order[pos] = row at position pos (-1 past the
+ * last kept row); counts [E] int64 = rows per expert before dropping; kept_counts [E] int64 = rows kept this
+ * round; within [n_rows] int32 optional.  workspace: picomoe_permute_workspace_bytes() bytes. */
+int64_t picomoe_permute_workspace_bytes(int64_t n_rows, int num_experts);
+int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
+                         int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts, int32_t* within, void* workspace,
+                         void* stream);
+
+/* Replaces the gathers tokens[token_idx] (EP/expert_parallel.py:216-217) and x[order] (:340) in one pass:
+ * out[i] = src[row_map[i] / div] for i < n_out (row_map NULL = identity, negative entries are skipped). */
+int picomoe_gather_rows(const void* src, const int32_t* row_map, int div, int64_t n_out, int64_t hidden, int dtype,
+                        void* out, void* stream);
+
+/* Replaces y_sorted[inv_order] + _combine_topk (EP/expert_parallel.py:341, :219-224) and the weighted index_add
+ * of EP/capacity_moe.py:158-160: out[t] = sum_j weights[t,j] * y[inv_order[t*top_k+j]] over the rows that were
+ * kept; products rounded to dtype, fp32 sum rounded once.  weights NULL = plain sum (the gradient of the
+ * expand/permute gather). */
+int picomoe_combine_fwd(const void* y, const int32_t* inv_order, const void* weights, int64_t n_tokens, int top_k,
+                        int64_t hidden, int dtype, void* out, void* stream);
+
+/* Backward of the above: d_y[inv_order[t*k+j]] = weights[t,j] * d_out[t]; d_weights[t,j] = <d_out[t], y[...]>
+ * (0 for dropped rows).  Rows of d_y that no kept row maps to are left untouched. */
+int picomoe_combine_bwd(const void* d_out, const void* y, const int32_t* inv_order, const void* weights, int64_t n_tokens,
+                        int top_k, int64_t hidden, int dtype, void* d_y, void* d_weights, void* stream);
+
+/* ---- Expert FFN: grouped SwiGLU GEMMs -----------------------------------------------------------------
+ * Rows are grouped by expert, expert e owning the next counts[e] rows (counts [E] int64 on the device, read by
+ * the kernels: no host copy).  n_rows = rows allocated in the row-major activations (>= sum of counts).
+ * gate_w / up_w [E, inter, hidden], down_w [E, hidden, inter], all contiguous, in dtype.  fp32 accumulation.
+ *
+ * picomoe_ffn_gate_up replaces the gate||up grouped GEMM + silu_and_mul (EP/megakernel.py:302-304;
+ * model.py:258): act [n_rows, inter] = silu(x . gate_w[e]^T) * (x . up_w[e]^T); inter13 [n_rows, 2*inter]
+ * (optional) receives [g | u] for the backward pass. */
+int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                        int64_t inter, const void* gate_w, const void* up_w, int dtype, void* act, void* inter13,
+                        void* stream);
+/* Replaces the down grouped GEMM with its optional row-weight epilogue (EP/megakernel.py:305, :95-96). */
+int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden, int64_t inter,
+                     const void* down_w, const void* row_weight, int dtype, void* y, void* stream);
+/* Replaces da = dy @ down_w[e] and _silu_and_mul_bwd (EP/megakernel.py:344-345, :187-197) in one kernel:
+ * d_inter13 [n_rows, 2*inter] = [dg | du]; act_out (optional) = silu(g) * u rebuilt from inter13. */
+int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                          int64_t inter, const void* down_w, const void* inter13, int dtype, void* d_inter13, void* act_out,
+                          void* stream);
+/* Replaces dx = d_inter13 @ w13[e] (EP/megakernel.py:346) without the concatenated w13. */
+int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                        int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx, void* stream);
+/* Replaces _grouped_wgrad (EP/megakernel.py:209-291): out [E, p_dim, q_dim] with out[e] = lhs_e^T @ rhs_e over the
+ * rows of expert e; lhs [n_rows, >=p_dim] with row stride ld_lhs, rhs likewise (so the two halves of d_inter13
+ * are addressed in place).  Empty experts get zeros. */
+int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, const int64_t* counts,
+                      int num_experts, int64_t n_rows, int64_t p_dim, int64_t q_dim, int dtype, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

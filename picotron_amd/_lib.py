@@ -25,8 +25,22 @@ _SIGNATURES = {
     "picomoe_error_string": [_i32],
     "picomoe_fp8_quant": [_p, _i32, _i64, _i64, _p, _p, _p],
     "picomoe_fp8_dequant": [_p, _p, _i64, _i64, _p, _i32, _p],
+    "picomoe_route_partials": [_i64, _i32],
+    "picomoe_route_fwd": [_p, _i32, _i64, _i32, _i32, _p, _i32, _p, _p, _p, _p, _p, _p],
+    "picomoe_route_bwd": [_p, _p, _p, _i32, _i64, _i32, _i32, _i32, _p, _p, _f32, _p, _p],
+    "picomoe_balance": [_p, _p, _i32, _i64, _i32, _i32, _f32, _f32, _p, _p, _p],
+    "picomoe_permute_workspace_bytes": [_i64, _i32],
+    "picomoe_permute_plan": [_p, _i64, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
+    "picomoe_gather_rows": [_p, _p, _i32, _i64, _i64, _i32, _p, _p],
+    "picomoe_combine_fwd": [_p, _p, _p, _i64, _i32, _i64, _i32, _p, _p],
+    "picomoe_combine_bwd": [_p, _p, _p, _p, _i64, _i32, _i64, _i32, _p, _p, _p],
+    "picomoe_ffn_gate_up": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
+    "picomoe_ffn_down": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p],
+    "picomoe_ffn_dgrad_act": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
+    "picomoe_ffn_dgrad_x": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p],
+    "picomoe_ffn_wgrad": [_p, _i64, _p, _i64, _p, _i32, _i64, _i64, _i64, _i32, _p, _p],
 }
-_RESTYPES = {"picomoe_error_string": ctypes.c_char_p}
+_RESTYPES = {"picomoe_error_string": ctypes.c_char_p, "picomoe_permute_workspace_bytes": ctypes.c_int64}
 
 _lib = None
 

@@ -1,0 +1,207 @@
+"""torch.autograd wrappers over the C-ABI kernels: router, permute plan, gather, combine.
+
+Host-side plumbing only (tensor allocation, stream, argument marshalling); all arithmetic is in
+``libpicomoe.so``.  Every function requires CUDA tensors.
+"""
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from picotron_amd import _lib
+
+
+def _empty(shape, dtype, device):
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
+# ------------------------------------------------------------------------------------------------
+# Router
+# ------------------------------------------------------------------------------------------------
+class _Route(torch.autograd.Function):
+    """softmax -> top-k -> gate weights (+ aux loss and loss-free bias step when ``balance``)."""
+
+    @staticmethod
+    def forward(ctx, logits, bias_f32, top_k, norm_topk, balance, aux_coef, bias_rate):
+        _lib.require_cuda(logits)
+        lib = _lib.load()
+        logits = logits.contiguous()
+        T, E = logits.shape
+        dev = logits.device
+        idx = _empty((T, top_k), torch.int64, dev)
+        w = _empty((T, top_k), logits.dtype, dev)
+        probs = _empty((T, E), torch.float32, dev)
+        counts = partial = None
+        n_part = 0
+        if balance:
+            counts = torch.zeros(E, dtype=torch.int32, device=dev)
+            if aux_coef > 0:
+                n_part = lib.picomoe_route_partials(T, E)
+                partial = _empty((n_part, E), torch.float32, dev)
+        _lib.check(
+            lib.picomoe_route_fwd(
+                _lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, top_k, _lib.ptr(bias_f32), int(bool(norm_topk)),
+                _lib.ptr(idx), _lib.ptr(w), _lib.ptr(probs), _lib.ptr(counts), _lib.ptr(partial), _lib.stream_ptr(),
+            ),
+            "picomoe_route_fwd",
+        )
+        aux = torch.zeros((), dtype=torch.float32, device=dev)
+        if balance and T > 0:
+            _lib.check(
+                lib.picomoe_balance(
+                    _lib.ptr(counts), _lib.ptr(partial), n_part, T, E, top_k, float(aux_coef), float(bias_rate),
+                    _lib.ptr(aux) if aux_coef > 0 else None, _lib.ptr(bias_f32) if bias_rate > 0 else None, _lib.stream_ptr(),
+                ),
+                "picomoe_balance",
+            )
+        ctx.save_for_backward(probs, idx, counts)
+        ctx.cfg = (top_k, bool(norm_topk), float(aux_coef) if balance else 0.0, logits.dtype)
+        ctx.mark_non_differentiable(idx)
+        return idx, w, aux
+
+    @staticmethod
+    def backward(ctx, _d_idx, d_w, d_aux):
+        probs, idx, counts = ctx.saved_tensors
+        top_k, norm, aux_coef, dtype = ctx.cfg
+        T, E = probs.shape
+        lib = _lib.load()
+        d_logits = _empty((T, E), dtype, probs.device)
+        d_w = d_w.contiguous() if d_w is not None else None
+        use_aux = aux_coef > 0 and d_aux is not None and counts is not None
+        d_aux = d_aux.contiguous().float() if use_aux else None
+        _lib.check(
+            lib.picomoe_route_bwd(
+                _lib.ptr(probs), _lib.ptr(idx), _lib.ptr(d_w), _lib.dtype_code(dtype), T, E, top_k, int(norm),
+                _lib.ptr(d_aux), _lib.ptr(counts) if use_aux else None, aux_coef, _lib.ptr(d_logits), _lib.stream_ptr(),
+            ),
+            "picomoe_route_bwd",
+        )
+        return d_logits, None, None, None, None, None, None
+
+
+def route(logits, bias_f32, top_k, norm_topk, balance=False, aux_coef=0.0, bias_rate=0.0):
+    """Returns (topk_idx int64 [T,k], topk_w [T,k] in logits.dtype, aux fp32 scalar)."""
+    return _Route.apply(logits, bias_f32, top_k, norm_topk, balance, aux_coef, bias_rate)
+
+
+# ------------------------------------------------------------------------------------------------
+# Permutation plan
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class Plan:
+    """Result of the stable counting sort of routed rows by expert (see include/picomoe.h)."""
+
+    order: torch.Tensor        # int32 [R]  row at each sorted position (-1 past the kept rows)
+    inv_order: torch.Tensor    # int32 [R]  sorted position of each row (-1 = dropped)
+    counts: torch.Tensor       # int64 [E]  rows per expert before any capacity limit
+    kept_counts: torch.Tensor  # int64 [E]  rows per expert in this plan's layout
+    within: Optional[torch.Tensor] = None  # int32 [R] rank of a row inside its expert
+    capacity: int = 0
+
+
+def permute_plan(expert_idx, num_experts, capacity=0, round_index=0, want_within=False):
+    _lib.require_cuda(expert_idx)
+    lib = _lib.load()
+    expert_idx = expert_idx.contiguous().to(torch.int64)
+    R = expert_idx.numel()
+    dev = expert_idx.device
+    order = _empty((R,), torch.int32, dev)
+    inv = _empty((R,), torch.int32, dev)
+    counts = _empty((num_experts,), torch.int64, dev)
+    kept = _empty((num_experts,), torch.int64, dev)
+    within = _empty((R,), torch.int32, dev) if want_within else None
+    ws_bytes = lib.picomoe_permute_workspace_bytes(R, num_experts)
+    if ws_bytes < 0:
+        raise _lib.PicomoeError(f"permute plan: unsupported size (rows={R}, experts={num_experts})")
+    ws = _empty((max(ws_bytes, 4),), torch.uint8, dev)
+    _lib.check(
+        lib.picomoe_permute_plan(
+            _lib.ptr(expert_idx), R, num_experts, int(capacity), int(round_index), _lib.ptr(order), _lib.ptr(inv),
+            _lib.ptr(counts), _lib.ptr(kept), _lib.ptr(within), _lib.ptr(ws), _lib.stream_ptr(),
+        ),
+        "picomoe_permute_plan",
+    )
+    return Plan(order, inv, counts, kept, within, int(capacity))
+
+
+# ------------------------------------------------------------------------------------------------
+# Row movers
+# ------------------------------------------------------------------------------------------------
+def gather_rows(src, row_map, div, n_out):
+    lib = _lib.load()
+    src = src.contiguous()
+    out = _empty((n_out, src.shape[1]), src.dtype, src.device)
+    _lib.check(
+        lib.picomoe_gather_rows(_lib.ptr(src), _lib.ptr(row_map), int(div), n_out, src.shape[1], _lib.dtype_code(src.dtype),
+                                _lib.ptr(out), _lib.stream_ptr()),
+        "picomoe_gather_rows",
+    )
+    return out
+
+
+def combine_rows(y, inv_order, weights, n_tokens, top_k):
+    lib = _lib.load()
+    y = y.contiguous()
+    weights = weights.contiguous() if weights is not None else None
+    out = _empty((n_tokens, y.shape[1]), y.dtype, y.device)
+    _lib.check(
+        lib.picomoe_combine_fwd(_lib.ptr(y), _lib.ptr(inv_order), _lib.ptr(weights), n_tokens, top_k, y.shape[1],
+                                _lib.dtype_code(y.dtype), _lib.ptr(out), _lib.stream_ptr()),
+        "picomoe_combine_fwd",
+    )
+    return out
+
+
+class _ExpandPermute(torch.autograd.Function):
+    """out[pos] = src[order[pos] // div]  (token-major expansion and the sort by expert in one gather).
+    Backward: d_src[t] = sum_j d_out[inv_order[t*div + j]] -- a gather-sum, no atomics."""
+
+    @staticmethod
+    def forward(ctx, src, order, inv_order, div, n_out):
+        _lib.require_cuda(src)
+        ctx.save_for_backward(inv_order)
+        ctx.meta = (src.shape[0], div)
+        return gather_rows(src, order, div, n_out)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        (inv_order,) = ctx.saved_tensors
+        n_src, div = ctx.meta
+        return combine_rows(d_out, inv_order, None, n_src, div), None, None, None, None
+
+
+def expand_permute(src, order, inv_order, div, n_out):
+    return _ExpandPermute.apply(src, order, inv_order, div, n_out)
+
+
+class _UnpermuteCombine(torch.autograd.Function):
+    """out[t] = sum_j w[t,j] * y[inv_order[t*k+j]] over kept rows (w None: k = 1 plain un-permute)."""
+
+    @staticmethod
+    def forward(ctx, y, weights, inv_order, order, n_tokens, top_k, zero_fill):
+        _lib.require_cuda(y)
+        ctx.save_for_backward(y, weights, inv_order, order)
+        ctx.meta = (n_tokens, top_k, zero_fill)
+        return combine_rows(y, inv_order, weights, n_tokens, top_k)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        y, weights, inv_order, order = ctx.saved_tensors
+        n_tokens, top_k, zero_fill = ctx.meta
+        d_out = d_out.contiguous()
+        if weights is None:
+            return gather_rows(d_out, order, 1, y.shape[0]), None, None, None, None, None, None
+        lib = _lib.load()
+        d_y = (torch.zeros if zero_fill else torch.empty)(y.shape, dtype=y.dtype, device=y.device)
+        d_w = _empty(weights.shape, weights.dtype, weights.device)
+        _lib.check(
+            lib.picomoe_combine_bwd(_lib.ptr(d_out), _lib.ptr(y), _lib.ptr(inv_order), _lib.ptr(weights), n_tokens, top_k,
+                                    y.shape[1], _lib.dtype_code(y.dtype), _lib.ptr(d_y), _lib.ptr(d_w), _lib.stream_ptr()),
+            "picomoe_combine_bwd",
+        )
+        return d_y, d_w, None, None, None, None, None
+
+
+def unpermute_combine(y, weights, inv_order, order, n_tokens, top_k, zero_fill=False):
+    return _UnpermuteCombine.apply(y, weights, inv_order, order, n_tokens, top_k, zero_fill)

@@ -1,0 +1,66 @@
+// extern "C" entry points of the expert FFN (grouped SwiGLU GEMMs, forward + dgrad + wgrad).
+// Picks the bf16 MFMA kernels when the shape is one they tile, the generic kernels otherwise.
+#include "ffn.h"
+
+namespace {
+bool fill_shape(FfnShape* s, const int64_t* counts, int E, int64_t n_rows, int64_t H, int64_t I, int dtype) {
+    if (!counts || E < 1 || E > 1024 || n_rows < 0 || n_rows >= (1ll << 31) || H < 1 || I < 1) return false;
+    if (dtype != PICOMOE_F32 && dtype != PICOMOE_BF16) return false;
+    s->counts = counts; s->E = E; s->n_rows = n_rows; s->H = H; s->I = I; s->dtype = dtype;
+    return true;
+}
+}  // namespace
+
+extern "C" int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                                   int64_t inter, const void* gate_w, const void* up_w, int dtype, void* act, void* inter13,
+                                   void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(x && gate_w && up_w && act);
+    if (ffn_mfma_supported(s)) return ffn_mfma_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
+    return ffn_simple_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
+}
+
+extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                                int64_t inter, const void* down_w, const void* row_weight, int dtype, void* y, void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(act && down_w && y);
+    if (ffn_mfma_supported(s)) return ffn_mfma_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
+    return ffn_simple_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
+}
+
+extern "C" int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
+                                     int64_t inter, const void* down_w, const void* inter13, int dtype, void* d_inter13,
+                                     void* act_out, void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(dy && down_w && inter13 && d_inter13);
+    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
+    return ffn_simple_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
+}
+
+extern "C" int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_experts, int64_t n_rows,
+                                   int64_t hidden, int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx,
+                                   void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(d_inter13 && gate_w && up_w && dx);
+    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
+    return ffn_simple_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
+}
+
+extern "C" int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, const int64_t* counts,
+                                 int num_experts, int64_t n_rows, int64_t p_dim, int64_t q_dim, int dtype, void* out,
+                                 void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, p_dim, q_dim, dtype));
+    PICOMOE_CHECK_ARG(lhs && rhs && out && ld_lhs >= p_dim && ld_rhs >= q_dim);
+    // n_rows == 0 still has to zero-fill the output: every expert is empty
+    if (ffn_mfma_supported(s)) return ffn_mfma_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
+    return ffn_simple_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
+}

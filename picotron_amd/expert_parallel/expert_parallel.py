@@ -1,0 +1,247 @@
+"""Mixture-of-Experts layer for one MI355X (all experts local, EP = 1).
+
+Drop-in for picotron/expert_parallel/expert_parallel.py: ``MoELayer`` (:38-439) keeps its constructor
+knobs, attributes, parameter names and private helpers (``_route`` :168, ``_balance`` folded into the
+router kernel, ``_expand_routed`` :214, ``_combine_topk`` :219, ``_moe_naive`` :271, ``_moe_capped`` :286,
+``_grouped_experts`` :311, ``_run_local_experts`` :331) and ``collect_aux_loss`` (:442-454).
+
+With one rank the dispatch / combine all-to-alls are local permutations, so the layer is:
+router kernel -> stable counting-sort plan -> one gather (expand + permute) -> grouped SwiGLU GEMMs ->
+one gather-sum (un-permute + gate-weighted combine).  The paths that exist only for several ranks
+(``_dispatch_combine``, ``_moe_tiled``, ``_moe_deepep``) have no counterpart here.
+Everything runs on the GPU through libpicomoe.so; CPU tensors are refused.
+"""
+
+import types
+
+import torch
+import torch.nn as nn
+
+from picotron_amd import _lib, _ops
+from picotron_amd.expert_parallel import megakernel
+from picotron_amd.expert_parallel.capacity_moe import _capped_rounds, compute_capacity
+from picotron_amd.expert_parallel.ep_communications import fp8_round_trip
+from picotron_amd.model import MLP
+
+
+def _argsort_inv(key, num_keys=None):
+    """Stable argsort by small integer keys plus its inverse permutation (``x[order][inv_order] == x``)."""
+    n = int(key.max().item()) + 1 if num_keys is None else num_keys
+    plan = _ops.permute_plan(key, n)
+    return plan.order.to(torch.int64), plan.inv_order.to(torch.int64)
+
+
+class _StackedWeights(torch.autograd.Function):
+    """Presents E per-expert parameters as one [E, ...] tensor without copying: ``stack`` already shares
+    storage with them.  Backward hands each parameter its slice of the stacked gradient."""
+
+    @staticmethod
+    def forward(ctx, stack, *params):
+        return stack.view_as(stack)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return (None, *grad.unbind(0))
+
+
+class MoELayer(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.num_experts = config.num_experts
+        self.top_k = config.num_experts_per_tok
+        self.norm_topk_prob = getattr(config, "norm_topk_prob", True)
+
+        # one GPU: every expert is local
+        self.ep_world_size = 1
+        self.ep_rank = 0
+        self.num_local_experts = self.num_experts
+
+        self.latent_dim = getattr(config, "moe_latent_dim", 0)
+        self.latent = 0 < self.latent_dim < self.hidden_size
+        self.expert_dim = self.latent_dim if self.latent else self.hidden_size
+
+        self.gate = nn.Linear(config.hidden_size, self.num_experts, bias=False)
+        if self.latent:
+            self.down_proj_latent = nn.Linear(self.hidden_size, self.latent_dim, bias=False)
+            self.up_proj_latent = nn.Linear(self.latent_dim, self.hidden_size, bias=False)
+        expert_config = types.SimpleNamespace(hidden_size=self.expert_dim, intermediate_size=config.intermediate_size)
+        self.local_experts = nn.ModuleList([MLP(expert_config) for _ in range(self.num_local_experts)])
+        self.num_shared_experts = getattr(config, "num_shared_experts", 0)
+        if self.num_shared_experts > 0:
+            shared_config = types.SimpleNamespace(
+                hidden_size=self.hidden_size, intermediate_size=config.intermediate_size * self.num_shared_experts
+            )
+            self.shared_expert = MLP(shared_config)
+        else:
+            self.shared_expert = None
+
+        # knobs of the multi-rank paths are kept as attributes (callers set them) but have no effect here
+        self.ep_overlap = getattr(config, "ep_overlap", True)
+        self.ep_num_tiles = getattr(config, "ep_num_tiles", 1)
+        self.ep_backend = getattr(config, "ep_backend", "torch")
+        self.ep_fp8_dispatch = getattr(config, "ep_fp8_dispatch", False)
+
+        self.ep_capacity_factor = getattr(config, "ep_capacity_factor", 0.0)
+        self.ep_capacity_dropless = getattr(config, "ep_capacity_dropless", True)
+        self.ep_max_rounds = getattr(config, "ep_max_rounds", 8)
+
+        self.router_aux_loss_coef = getattr(config, "router_aux_loss_coef", 0.0)
+        self.router_bias_update_rate = getattr(config, "router_bias_update_rate", 0.0)
+        self.use_loss_free = self.router_bias_update_rate > 0
+        self.register_buffer("expert_bias", torch.zeros(self.num_experts), persistent=True)
+        self.aux_loss = None
+
+        self._stacks = None  # [E,I,H], [E,I,H], [E,H,I] buffers the per-expert parameters are views of
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.gate.reset_parameters()
+        if self.latent:
+            self.down_proj_latent.reset_parameters()
+            self.up_proj_latent.reset_parameters()
+        for expert in self.local_experts:
+            expert.reset_parameters()
+        if self.shared_expert is not None:
+            self.shared_expert.reset_parameters()
+
+    # ---- expert weights as stacked tensors ------------------------------------------------------
+    def _expert_params(self):
+        ex = self.local_experts
+        return ([e.gate_proj.weight for e in ex], [e.up_proj.weight for e in ex], [e.down_proj.weight for e in ex])
+
+    def _stacked_weights(self):
+        """(gate_w [E,I,H], up_w [E,I,H], down_w [E,H,I]) sharing storage with the per-expert parameters.
+
+        The first call (and any call after the parameters were moved, cast or re-assigned) copies the
+        weights once into three contiguous buffers and re-points every ``local_experts[i].*_proj.weight``
+        at its slice; afterwards optimizer steps and ``load_state_dict`` update the buffers in place and
+        no per-forward ``stack`` is needed."""
+        groups = self._expert_params()
+        p0 = groups[0][0]
+        ok = self._stacks is not None and all(s.dtype == p0.dtype and s.device == p0.device for s in self._stacks)
+        if ok:
+            for stack, params in zip(self._stacks, groups):
+                step = stack.stride(0) * stack.element_size()
+                base = stack.data_ptr()
+                if any(p.data_ptr() != base + i * step or p.shape != stack.shape[1:] for i, p in enumerate(params)):
+                    ok = False
+                    break
+        if not ok:
+            with torch.no_grad():
+                stacks = []
+                for params in groups:
+                    stack = torch.stack([p.detach() for p in params]).contiguous()
+                    for i, p in enumerate(params):
+                        p.data = stack[i]
+                    stacks.append(stack)
+                self._stacks = tuple(stacks)
+        return tuple(_StackedWeights.apply(stack, *params) for stack, params in zip(self._stacks, groups))
+
+    # ---- forward ----------------------------------------------------------------------------------
+    def forward(self, x):
+        batch_size, seq_length, _ = x.shape
+        tokens = x.reshape(-1, self.hidden_size)
+        topk_idx, topk_weights = self._route(tokens)
+        if self.ep_capacity_factor > 0:
+            expert_out = self._moe_capped(tokens, topk_idx, topk_weights)
+        else:
+            expert_out = self._moe_naive(tokens, topk_idx, topk_weights)
+        return expert_out.view(batch_size, seq_length, self.hidden_size)
+
+    def _route(self, tokens):
+        """Router: top-k expert selection + gate weights; stashes the aux loss and steps the loss-free bias
+        (training only), all inside the router kernels."""
+        _lib.require_cuda(tokens)
+        router_logits = self.gate(tokens)
+        balance = self.training and (self.router_aux_loss_coef > 0 or self.use_loss_free)
+        # fp32 view or copy of the bias: the router kernel reads it for the selection, the balance kernel that
+        # follows on the same stream steps it in place
+        bias_f32 = self.expert_bias.float() if self.use_loss_free else None
+        topk_idx, topk_weights, aux = _ops.route(
+            router_logits, bias_f32, self.top_k, self.norm_topk_prob, balance,
+            self.router_aux_loss_coef if balance else 0.0, self.router_bias_update_rate if (balance and self.use_loss_free) else 0.0,
+        )
+        self.aux_loss = aux if (balance and self.router_aux_loss_coef > 0) else None
+        if balance and self.use_loss_free:
+            with torch.no_grad():
+                self.expert_bias.copy_(bias_f32)
+        return topk_idx, topk_weights
+
+    def _expand_routed(self, tokens, topk_idx, topk_weights):
+        """One routed row per (token, selected expert), token-major."""
+        n = tokens.shape[0] * self.top_k
+        return _ops.expand_permute(tokens, None, None, self.top_k, n), topk_idx.reshape(-1), topk_weights.reshape(-1)
+
+    def _combine_topk(self, y, weights, num_tokens):
+        """Weight each routed row by its gate weight and sum a token's top-k rows."""
+        return _ops.unpermute_combine(y, weights.reshape(num_tokens, self.top_k), None, None, num_tokens, self.top_k)
+
+    def _maybe_down(self, tokens):
+        return self.down_proj_latent(tokens) if self.latent else tokens
+
+    def _shared_start(self, tokens):
+        if self.shared_expert is None:
+            return None, None
+        return self.shared_expert(tokens), None
+
+    def _finalize(self, y_expert, shared):
+        y = self.up_proj_latent(y_expert) if self.latent else y_expert
+        shared_out, _ = shared
+        return y if shared_out is None else y + shared_out
+
+    def _moe_naive(self, tokens, topk_idx, topk_weights):
+        _lib.require_cuda(tokens, topk_idx, topk_weights)
+        num_tokens = tokens.shape[0]
+        shared = self._shared_start(tokens)
+        latent = self._maybe_down(tokens)
+        if self.ep_fp8_dispatch:
+            # one quantise -> dequantise per token equals one per routed row (a row op on identical rows)
+            latent = fp8_round_trip(latent)
+        n_rows = num_tokens * self.top_k
+        plan = _ops.permute_plan(topk_idx.reshape(-1), self.num_local_experts)
+        x_sorted = _ops.expand_permute(latent, plan.order, plan.inv_order, self.top_k, n_rows)
+        y_sorted = self._grouped_experts(x_sorted, plan.counts)
+        y = _ops.unpermute_combine(y_sorted, topk_weights, plan.inv_order, plan.order, num_tokens, self.top_k)
+        return self._finalize(y, shared)
+
+    def _moe_capped(self, tokens, topk_idx, topk_weights):
+        """MoE under a fixed per-expert capacity: one round with drops, or dropless rounds (see capacity_moe.py)."""
+        _lib.require_cuda(tokens, topk_idx, topk_weights)
+        num_tokens = tokens.shape[0]
+        shared = self._shared_start(tokens)
+        latent = self._maybe_down(tokens)
+        capacity = compute_capacity(num_tokens, self.top_k, self.num_experts, self.ep_capacity_factor)
+        y, _ = _capped_rounds(
+            latent, self.top_k, topk_idx.reshape(-1), topk_weights, num_tokens, self.top_k, self.num_experts,
+            self._grouped_experts, capacity, self.ep_capacity_dropless, self.ep_max_rounds,
+        )
+        return self._finalize(y, shared)
+
+    def _grouped_experts(self, x_sorted, counts):
+        """Run the local experts on rows already grouped by expert; ``counts[e]`` rows go to expert ``e``."""
+        if x_sorted.shape[0] == 0:
+            return x_sorted
+        _lib.require_cuda(x_sorted)
+        gate_w, up_w, down_w = self._stacked_weights()
+        return megakernel.fused_moe(x_sorted, counts, gate_w, up_w, down_w)
+
+    def _run_local_experts(self, x, local_expert_idx):
+        """Run the local experts on ``x`` given each row's expert id, preserving the input order."""
+        if x.shape[0] == 0:
+            return x
+        n = x.shape[0]
+        plan = _ops.permute_plan(local_expert_idx, self.num_local_experts)
+        x_sorted = _ops.expand_permute(x, plan.order, plan.inv_order, 1, n)
+        y_sorted = self._grouped_experts(x_sorted, plan.counts)
+        return _ops.unpermute_combine(y_sorted, None, plan.inv_order, plan.order, n, 1)
+
+
+def collect_aux_loss(model):
+    """Sum and drain the aux loss stashed on every ``MoELayer`` by its last forward (``None`` if there is none)."""
+    total = None
+    for module in model.modules():
+        if isinstance(module, MoELayer) and module.aux_loss is not None:
+            total = module.aux_loss if total is None else total + module.aux_loss
+            module.aux_loss = None
+    return total

@@ -1,0 +1,223 @@
+"""Expert FFN (grouped SwiGLU GEMMs) on hand-written gfx950 kernels.
+
+Same public surface as picotron/expert_parallel/megakernel.py: ``fused_moe`` (:403),
+``fused_moe_forward`` (:294), ``fused_moe_dgrad`` (:332), ``fused_moe_wgrad`` (:350),
+``fused_moe_backward`` (:360), ``torch_fused_ffn`` (:308), ``torch_moe_backward`` (:321),
+``cuda_available`` (:408).  ``x_sorted [N,H]`` holds rows grouped by expert, ``counts [E]`` is a device
+tensor read by the kernels (no host copy, no block schedule built on the host), ``gate_w/up_w [E,I,H]``,
+``down_w [E,H,I]``.
+
+Differences in mechanism, not in results: gate and up are consumed in place (no ``cat`` into w13), SwiGLU
+is the epilogue of the gate/up GEMM, silu-mul-backward is the epilogue of the ``dy @ down_w`` GEMM, and the
+autograd path keeps ``[g|u]`` from the forward instead of recomputing it.
+"""
+
+import torch
+import torch.nn.functional as F
+
+from picotron_amd import _lib
+
+
+def cuda_available():
+    """Whether the HIP kernels can run: a GPU is visible and libpicomoe.so loads."""
+    if not torch.cuda.is_available():
+        return False
+    _lib.load()
+    return True
+
+
+def _counts64(counts, device):
+    if not torch.is_tensor(counts):
+        counts = torch.tensor(list(counts), dtype=torch.int64, device=device)
+    return counts.to(device=device, dtype=torch.int64).contiguous()
+
+
+def _check_weights(x, gate_w, up_w, down_w):
+    E, I, H = gate_w.shape
+    if up_w.shape != (E, I, H) or down_w.shape != (E, H, I) or x.shape[1] != H:
+        raise _lib.PicomoeError(f"fused_moe: shapes x{tuple(x.shape)} gate{tuple(gate_w.shape)} up{tuple(up_w.shape)} down{tuple(down_w.shape)}")
+    if not (x.dtype == gate_w.dtype == up_w.dtype == down_w.dtype):
+        raise _lib.PicomoeError("fused_moe: x and the weights must share one dtype")
+    return E, I, H
+
+
+def _gate_up(x, counts, gate_w, up_w, keep_inter13):
+    lib = _lib.load()
+    E, I, H = gate_w.shape
+    N = x.shape[0]
+    act = torch.empty((N, I), dtype=x.dtype, device=x.device)
+    inter13 = torch.empty((N, 2 * I), dtype=x.dtype, device=x.device) if keep_inter13 else None
+    _lib.check(
+        lib.picomoe_ffn_gate_up(_lib.ptr(x), _lib.ptr(counts), E, N, H, I, _lib.ptr(gate_w), _lib.ptr(up_w),
+                                _lib.dtype_code(x.dtype), _lib.ptr(act), _lib.ptr(inter13), _lib.stream_ptr()),
+        "picomoe_ffn_gate_up",
+    )
+    return act, inter13
+
+
+def _down(act, counts, down_w, row_weight):
+    lib = _lib.load()
+    E, H, I = down_w.shape
+    N = act.shape[0]
+    y = torch.empty((N, H), dtype=act.dtype, device=act.device)
+    _lib.check(
+        lib.picomoe_ffn_down(_lib.ptr(act), _lib.ptr(counts), E, N, H, I, _lib.ptr(down_w), _lib.ptr(row_weight),
+                             _lib.dtype_code(act.dtype), _lib.ptr(y), _lib.stream_ptr()),
+        "picomoe_ffn_down",
+    )
+    return y
+
+
+def _dgrad_act(dy, counts, down_w, inter13, want_act):
+    lib = _lib.load()
+    E, H, I = down_w.shape
+    N = dy.shape[0]
+    d13 = torch.empty((N, 2 * I), dtype=dy.dtype, device=dy.device)
+    act = torch.empty((N, I), dtype=dy.dtype, device=dy.device) if want_act else None
+    _lib.check(
+        lib.picomoe_ffn_dgrad_act(_lib.ptr(dy), _lib.ptr(counts), E, N, H, I, _lib.ptr(down_w), _lib.ptr(inter13),
+                                  _lib.dtype_code(dy.dtype), _lib.ptr(d13), _lib.ptr(act), _lib.stream_ptr()),
+        "picomoe_ffn_dgrad_act",
+    )
+    return d13, act
+
+
+def _dgrad_x(d13, counts, gate_w, up_w):
+    lib = _lib.load()
+    E, I, H = gate_w.shape
+    N = d13.shape[0]
+    dx = torch.empty((N, H), dtype=d13.dtype, device=d13.device)
+    _lib.check(
+        lib.picomoe_ffn_dgrad_x(_lib.ptr(d13), _lib.ptr(counts), E, N, H, I, _lib.ptr(gate_w), _lib.ptr(up_w),
+                                _lib.dtype_code(d13.dtype), _lib.ptr(dx), _lib.stream_ptr()),
+        "picomoe_ffn_dgrad_x",
+    )
+    return dx
+
+
+def _wgrad(lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset=0):
+    lib = _lib.load()
+    out = torch.empty((E, P, Q), dtype=dtype, device=device)
+    lhs_ptr = _lib.ctypes.c_void_p(lhs.data_ptr() + lhs_offset * lhs.element_size())
+    _lib.check(
+        lib.picomoe_ffn_wgrad(lhs_ptr, ld_lhs, _lib.ptr(rhs), ld_rhs, _lib.ptr(counts), E, N, P, Q, _lib.dtype_code(dtype),
+                              _lib.ptr(out), _lib.stream_ptr()),
+        "picomoe_ffn_wgrad",
+    )
+    return out
+
+
+def _prep(x_sorted, counts, *weights):
+    _lib.require_cuda(x_sorted, *weights)
+    return x_sorted.contiguous(), _counts64(counts, x_sorted.device), [w.contiguous() for w in weights]
+
+
+def fused_moe_forward(x_sorted, counts, gate_w, up_w, down_w, row_weight=None):
+    """x_sorted [N,H] (rows grouped by expert); gate_w/up_w [E,I,H]; down_w [E,H,I]; counts [E]."""
+    x, counts, (gw, uw, dw) = _prep(x_sorted, counts, gate_w, up_w, down_w)
+    _check_weights(x, gw, uw, dw)
+    if x.shape[0] == 0:
+        return torch.empty((0, x.shape[1]), device=x.device, dtype=x.dtype)
+    act, _ = _gate_up(x, counts, gw, uw, keep_inter13=False)
+    rw = row_weight.to(x.dtype).contiguous() if row_weight is not None else None
+    return _down(act, counts, dw, rw)
+
+
+def fused_moe_dgrad(x_sorted, counts, gate_w, up_w, down_w, dy):
+    """Explicit input-grad.  Returns (dx, a, d_inter13); ``a`` / ``d_inter13`` feed ``fused_moe_wgrad``.
+    Stateless like the reference: the forward intermediates are rebuilt here."""
+    x, counts, (gw, uw, dw) = _prep(x_sorted, counts, gate_w, up_w, down_w)
+    dy = dy.contiguous()
+    act, inter13 = _gate_up(x, counts, gw, uw, keep_inter13=True)
+    d13, _ = _dgrad_act(dy, counts, dw, inter13, want_act=False)
+    dx = _dgrad_x(d13, counts, gw, uw)
+    return dx, act, d13
+
+
+def fused_moe_wgrad(x_sorted, counts, a, d_inter13, dy):
+    """Explicit weight-grads from the forward intermediates.  Returns (d_gate, d_up, d_down)."""
+    _lib.require_cuda(x_sorted, a, d_inter13, dy)
+    x, a, d13, dy = x_sorted.contiguous(), a.contiguous(), d_inter13.contiguous(), dy.contiguous()
+    counts = _counts64(counts, x.device)
+    E, N, H, I = counts.numel(), x.shape[0], x.shape[1], a.shape[1]
+    d_down = _wgrad(dy, H, a, I, counts, E, N, H, I, x.dtype, x.device)
+    d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
+    d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
+    return d_gate, d_up, d_down
+
+
+def fused_moe_backward(x_sorted, counts, gate_w, up_w, down_w, dy):
+    """(dx, d_gate, d_up, d_down) with explicit dgrad + wgrad kernels."""
+    if x_sorted.shape[0] == 0:
+        return (torch.zeros_like(x_sorted), torch.zeros_like(gate_w), torch.zeros_like(up_w), torch.zeros_like(down_w))
+    dx, a, d13 = fused_moe_dgrad(x_sorted, counts, gate_w, up_w, down_w, dy)
+    d_gate, d_up, d_down = fused_moe_wgrad(x_sorted, counts, a, d13, dy)
+    return dx, d_gate, d_up, d_down
+
+
+class _FusedMoE(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x_sorted, gate_w, up_w, down_w, counts, row_weight):
+        x, counts, (gw, uw, dw) = _prep(x_sorted, counts, gate_w, up_w, down_w)
+        _check_weights(x, gw, uw, dw)
+        ctx.counts = counts
+        ctx.has_rw = row_weight is not None
+        if x.shape[0] == 0:
+            ctx.empty = True
+            ctx.save_for_backward(x, gw, uw, dw)
+            return torch.empty((0, x.shape[1]), device=x.device, dtype=x.dtype)
+        ctx.empty = False
+        needs_grad = any(ctx.needs_input_grad[:4]) or (ctx.has_rw and ctx.needs_input_grad[5])
+        act, inter13 = _gate_up(x, counts, gw, uw, keep_inter13=needs_grad)
+        rw = row_weight.to(x.dtype).contiguous() if ctx.has_rw else None
+        y = _down(act, counts, dw, rw)
+        if needs_grad:
+            ctx.save_for_backward(x, gw, uw, dw, act, inter13, rw)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        if ctx.empty:
+            x, gw, uw, dw = ctx.saved_tensors
+            return torch.zeros_like(x), torch.zeros_like(gw), torch.zeros_like(uw), torch.zeros_like(dw), None, None
+        x, gw, uw, dw, act, inter13, rw = ctx.saved_tensors
+        counts = ctx.counts
+        dy = grad_y.contiguous()
+        d_rw = None
+        if rw is not None:
+            # y = y0 * rw: d_rw = <dy, y0>, d_y0 = dy * rw  (y0 rebuilt by one more down GEMM)
+            y0 = _down(act, counts, dw, None)
+            d_rw = (dy.float() * y0.float()).sum(dim=1).to(rw.dtype)
+            dy = dy * rw[:, None]
+        d13, _ = _dgrad_act(dy, counts, dw, inter13, want_act=False)
+        dx = _dgrad_x(d13, counts, gw, uw)
+        E, N, H, I = counts.numel(), x.shape[0], x.shape[1], act.shape[1]
+        d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device)
+        d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
+        d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
+        return dx, d_gate, d_up, d_down, None, d_rw
+
+
+def fused_moe(x_sorted, counts, gate_w, up_w, down_w, row_weight=None):
+    """Differentiable fused MoE expert FFN.  counts [E] = per-expert row counts."""
+    return _FusedMoE.apply(x_sorted, gate_w, up_w, down_w, counts, row_weight)
+
+
+def torch_fused_ffn(x_sorted, counts, gate_w, up_w, down_w, row_weight):
+    """Per-expert loop over library matmuls, kept because the reference exposes it by name
+    (megakernel.py:308-318).  Nothing in this package dispatches to it."""
+    outs, offset = [], 0
+    for e, n in enumerate(counts.tolist()):
+        x = x_sorted[offset : offset + n]
+        outs.append((F.silu(x @ gate_w[e].T) * (x @ up_w[e].T)) @ down_w[e].T)
+        offset += n
+    y = torch.cat(outs, dim=0) if outs else x_sorted.new_empty((0, x_sorted.shape[1]))
+    return y * row_weight[:, None] if row_weight is not None else y
+
+
+def torch_moe_backward(x_sorted, counts, gate_w, up_w, down_w, dy):
+    """Autograd over ``torch_fused_ffn`` (megakernel.py:321-329); exposed by name only, never dispatched to."""
+    with torch.enable_grad():
+        leaves = [t.detach().requires_grad_(True) for t in (x_sorted, gate_w, up_w, down_w)]
+        y = torch_fused_ffn(leaves[0], counts, leaves[1], leaves[2], leaves[3], None)
+        return torch.autograd.grad(y, leaves, dy)

@@ -1,0 +1,138 @@
+"""GPU parity of the expert FFN (grouped SwiGLU GEMMs, forward / dgrad / wgrad) against the CPU oracle.
+
+Shapes and tolerances of the first three tests are the ones the reference's own kernel test uses
+(tests/test_megakernel.py:29-99): ragged counts with an empty expert and one longer than a tile,
+fp32 atol = rtol = 1e-4 forward and 1e-3 on gradients, the row-weight epilogue, bf16 max |diff| < 5e-2.
+"""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(E, H, I, counts, dtype, seed, scale=0.1):
+    g = torch.Generator().manual_seed(seed)
+    N = int(sum(counts))
+    x = torch.randn(N, H, generator=g).to(dtype)
+    gw = (torch.randn(E, I, H, generator=g) * scale).to(dtype)
+    uw = (torch.randn(E, I, H, generator=g) * scale).to(dtype)
+    dw = (torch.randn(E, H, I, generator=g) * scale).to(dtype)
+    return x, torch.tensor(counts, dtype=torch.int64), gw, uw, dw, g
+
+
+def test_fwd_bwd_ragged_fp32(gpu):
+    from picotron_amd.expert_parallel import megakernel
+
+    x, counts, gw, uw, dw, g = _mk(4, 48, 96, [5, 0, 130, 17], torch.float32, 0)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw)]
+    y = megakernel.fused_moe(leaves[0], counts.cuda(), *leaves[1:])
+    yr = O.expert_ffn(x, counts, gw, uw, dw)
+    assert torch.allclose(y.cpu(), yr, atol=1e-4, rtol=1e-4)
+    assert (y.cpu() - yr).abs().max() <= 1e-5 * yr.abs().max()        # and the fp32 bar of this build
+    dy = torch.randn(y.shape, generator=g)
+    y.backward(dy.cuda())
+    ref = O.expert_ffn_backward(x, counts, gw, uw, dw, dy)
+    for got, want, name in zip([l.grad for l in leaves], ref, ("dx", "dgate", "dup", "ddown")):
+        d = (got.cpu() - want).abs().max().item()
+        assert d < 1e-3, (name, d)
+        assert d <= 1e-5 * want.abs().max().item() + 1e-7, (name, d)
+    assert torch.all(leaves[1].grad[1] == 0) and torch.all(leaves[3].grad[1] == 0)   # the empty expert
+
+
+def test_row_weight_epilogue(gpu):
+    from picotron_amd.expert_parallel import megakernel
+
+    x, counts, gw, uw, dw, g = _mk(3, 32, 64, [20, 33, 7], torch.float32, 1)
+    rw = torch.rand(60, generator=g)
+    y = megakernel.fused_moe(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda(), row_weight=rw.cuda())
+    yr = O.expert_ffn(x, counts, gw, uw, dw, rw)
+    assert torch.allclose(y.cpu(), yr, atol=1e-4)
+    # and its gradient, including d row_weight
+    leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw, rw)]
+    yy = megakernel.fused_moe(leaves[0], counts.cuda(), leaves[1], leaves[2], leaves[3], row_weight=leaves[4])
+    dy = torch.randn(yy.shape, generator=g)
+    yy.backward(dy.cuda())
+    cl = [t.clone().requires_grad_(True) for t in (x, gw, uw, dw, rw)]
+    O.expert_ffn(cl[0], counts, cl[1], cl[2], cl[3], cl[4]).backward(dy)
+    for a, b in zip(leaves, cl):
+        assert torch.allclose(a.grad.cpu(), b.grad, atol=1e-4, rtol=1e-4)
+
+
+def test_bf16_small(gpu):
+    from picotron_amd.expert_parallel import megakernel
+
+    x, counts, gw, uw, dw, _ = _mk(4, 64, 128, [16, 16, 16, 16], torch.bfloat16, 2)
+    y = megakernel.fused_moe(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda())
+    yr = O.expert_ffn(x, counts, gw, uw, dw)
+    assert (y.cpu().float() - yr.float()).abs().max().item() < 5e-2
+
+
+def test_empty_input_and_all_empty_but_one(gpu):
+    from picotron_amd.expert_parallel import megakernel
+
+    x, counts, gw, uw, dw, _ = _mk(3, 16, 32, [0, 0, 0], torch.float32, 3)
+    y = megakernel.fused_moe(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda())
+    assert y.shape == (0, 16)
+    grads = megakernel.fused_moe_backward(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda(), y)
+    assert all(torch.all(t == 0) for t in grads) and grads[1].shape == gw.shape
+    x, counts, gw, uw, dw, _ = _mk(3, 16, 32, [0, 0, 9], torch.float32, 4)
+    y = megakernel.fused_moe_forward(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda())
+    assert torch.allclose(y.cpu(), O.expert_ffn(x, counts, gw, uw, dw), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_explicit_dgrad_wgrad_api(gpu, dtype):
+    """fused_moe_dgrad / fused_moe_wgrad return the intermediates the reference documents (a, d_inter13)."""
+    from picotron_amd.expert_parallel import megakernel
+
+    E, H, I = 3, 40, 72
+    x, counts, gw, uw, dw, g = _mk(E, H, I, [33, 0, 70], dtype, 5)
+    dy = torch.randn(x.shape, generator=g).to(dtype)
+    dx, a, d13 = megakernel.fused_moe_dgrad(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda(), dy.cuda())
+    dg, du, dd = megakernel.fused_moe_wgrad(x.cuda(), counts.cuda(), a, d13, dy.cuda())
+    xf, gf, uf, df, dyf = (t.float() for t in (x, gw, uw, dw, dy))
+    rdx, rdg, rdu, rdd = O.expert_ffn_backward(xf, counts, gf, uf, df, dyf)
+    # intermediates from their definitions
+    owner = torch.repeat_interleave(torch.arange(E), counts)
+    g13 = torch.cat([torch.einsum("nh,nih->ni", xf, gf[owner]), torch.einsum("nh,nih->ni", xf, uf[owner])], 1)
+    ra = torch.nn.functional.silu(g13[:, :I]) * g13[:, I:]
+    rd13 = O.silu_and_mul_bwd(g13, torch.einsum("nh,nhi->ni", dyf, df[owner]))
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=5e-2, atol=5e-2)
+    for got, want in ((dx, rdx), (a, ra), (d13, rd13), (dg, rdg), (du, rdu), (dd, rdd)):
+        assert torch.allclose(got.cpu().float(), want, **tol)
+
+
+@pytest.mark.parametrize("H,I,counts", [(256, 512, [130, 128, 126, 0, 1, 64, 63, 0]), (100, 36, [7, 300])])
+def test_bf16_ragged_against_oracle(gpu, H, I, counts):
+    """bf16: outputs and gradients within rtol 1e-2 of the oracle (measured against the magnitude of each tensor)."""
+    from picotron_amd.expert_parallel import megakernel
+
+    E = len(counts)
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.bfloat16, 6, scale=0.05)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw)]
+    y = megakernel.fused_moe(leaves[0], cnt.cuda(), *leaves[1:])
+    yr = O.expert_ffn(x, cnt, gw, uw, dw)
+    assert (y.cpu().float() - yr.float()).abs().max() <= 1e-2 * yr.float().abs().max()
+    dy = torch.randn(y.shape, generator=g).bfloat16()
+    y.backward(dy.cuda())
+    ref = O.expert_ffn_backward(x.float(), cnt, gw.float(), uw.float(), dw.float(), dy.float())
+    for got, want in zip([l.grad for l in leaves], ref):
+        assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
+
+
+def test_mlp_module_runs_the_kernels(gpu):
+    import types
+
+    from picotron_amd.model import MLP
+
+    torch.manual_seed(0)
+    m = MLP(types.SimpleNamespace(hidden_size=32, intermediate_size=80)).cuda()
+    x = torch.randn(3, 5, 32)
+    y = m(x.cuda())
+    want = O.mlp(x, m.gate_proj.weight.detach().cpu(), m.up_proj.weight.detach().cpu(), m.down_proj.weight.detach().cpu())
+    assert y.shape == (3, 5, 32) and torch.allclose(y.cpu(), want, atol=1e-5)
+    y.sum().backward()
+    assert all(p.grad is not None for p in m.parameters())

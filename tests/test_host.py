@@ -1,0 +1,100 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol include/picomoe.h declares, host
+logic (capacity, module structure, refusal of CPU tensors).  No kernels run here."""
+
+import os
+import re
+import types
+
+import pytest
+import torch
+
+from picotron_amd import _lib
+
+
+def _declared_symbols():
+    text = open(_lib.HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(picomoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 18
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert set(_lib.exported_symbols()) == set(declared)      # the ctypes table and the header agree
+    assert lib.picomoe_abi_version() == _lib.ABI_VERSION
+    assert b"unsupported" in lib.picomoe_error_string(1)
+    assert lib.picomoe_error_string(0) == b"ok"
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    lib = _lib.load()
+    null = None
+    assert lib.picomoe_fp8_quant(null, 7, 4, 8, null, null, null) == 1           # bad dtype
+    assert lib.picomoe_fp8_quant(null, 1, 4, 0, null, null, null) == 1           # bad width
+    assert lib.picomoe_fp8_quant(null, 1, 0, 8, null, null, null) == 0           # empty input is fine
+    assert lib.picomoe_route_fwd(null, 1, 4, 2000, 2, null, 1, null, null, null, null, null, null) == 1   # too many experts
+    assert lib.picomoe_route_fwd(null, 1, 4, 8, 9, null, 1, null, null, null, null, null, null) == 1      # top_k > E
+    assert lib.picomoe_permute_workspace_bytes(1000, 8) > 0
+    assert lib.picomoe_permute_workspace_bytes(1000, 5000) == -1
+    assert lib.picomoe_route_partials(8192, 8) >= 1
+    with pytest.raises(_lib.PicomoeError):
+        _lib.check(1, "demo")
+
+
+def test_compute_capacity_matches_reference_table():
+    from picotron_amd.expert_parallel.capacity_moe import compute_capacity
+
+    assert [compute_capacity(512, 2, 8, f) for f in (0.5, 1.0, 1.25, 2.0)] == [64, 128, 160, 256]
+    assert compute_capacity(16384, 6, 64, 1.25) == 1920
+    assert compute_capacity(3, 1, 64, 0.1) == 1
+
+
+def _cfg(**kw):
+    base = dict(hidden_size=16, intermediate_size=32, num_experts=4, num_experts_per_tok=2)
+    base.update(kw)
+    return types.SimpleNamespace(**base)
+
+
+def test_module_structure_and_defaults():
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer, collect_aux_loss
+
+    moe = MoELayer(_cfg(num_shared_experts=2, moe_latent_dim=8, router_bias_update_rate=0.01))
+    assert moe.expert_dim == 8 and moe.latent and moe.use_loss_free
+    assert moe.local_experts[0].gate_proj.weight.shape == (32, 8)
+    assert moe.shared_expert.gate_proj.weight.shape == (64, 16)
+    assert moe.down_proj_latent.weight.shape == (8, 16) and moe.up_proj_latent.weight.shape == (16, 8)
+    assert moe.expert_bias.shape == (4,) and "expert_bias" in moe.state_dict()
+    plain = MoELayer(_cfg())
+    assert plain.shared_expert is None and not plain.latent and plain.norm_topk_prob
+    assert (plain.ep_capacity_factor, plain.ep_capacity_dropless, plain.ep_max_rounds) == (0.0, True, 8)
+    assert plain.ep_fp8_dispatch is False and plain.router_aux_loss_coef == 0.0 and plain.aux_loss is None
+    assert plain.ep_world_size == 1 and plain.num_local_experts == 4
+    assert collect_aux_loss(plain) is None
+    # default init: uniform in +-1/sqrt(fan_in), like the reference MLP
+    w = plain.local_experts[0].down_proj.weight
+    assert w.abs().max() <= (1.0 / 32) ** 0.5
+
+
+def test_cpu_tensors_are_refused_not_silently_computed():
+    from picotron_amd.expert_parallel import megakernel
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer
+
+    moe = MoELayer(_cfg())
+    with pytest.raises(_lib.PicomoeError):
+        moe(torch.randn(1, 4, 16))
+    with pytest.raises(_lib.PicomoeError):
+        megakernel.fused_moe(torch.randn(4, 16), torch.tensor([4]), torch.randn(1, 32, 16), torch.randn(1, 32, 16), torch.randn(1, 16, 32))
+    if not torch.cuda.is_available():
+        assert megakernel.cuda_available() is False
+
+
+def test_product_does_not_import_the_oracle():
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dirpath, _, files in os.walk(os.path.join(root, "picotron_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower() or f == "README.md", os.path.join(dirpath, f)
