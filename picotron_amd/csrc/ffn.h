@@ -30,6 +30,7 @@ int ffn_simple_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const v
 
 // bf16 MFMA family: each returns PICOMOE_ERR_ARG without launching when the shape is not one it handles.
 bool ffn_mfma_supported(const FfnShape& s);
+bool ffn_mfma_wgrad_supported(int dtype, int64_t P, int64_t Q, int64_t ld_lhs, int64_t ld_rhs, const void* lhs, const void* rhs);
 int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
                      hipStream_t st);
 int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, hipStream_t st);

@@ -61,6 +61,7 @@ extern "C" int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rh
     PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, p_dim, q_dim, dtype));
     PICOMOE_CHECK_ARG(lhs && rhs && out && ld_lhs >= p_dim && ld_rhs >= q_dim);
     // n_rows == 0 still has to zero-fill the output: every expert is empty
-    if (ffn_mfma_supported(s)) return ffn_mfma_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
+    if (ffn_mfma_wgrad_supported(dtype, p_dim, q_dim, ld_lhs, ld_rhs, lhs, rhs))
+        return ffn_mfma_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
     return ffn_simple_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
 }

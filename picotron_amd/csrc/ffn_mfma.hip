@@ -1,65 +1,97 @@
 // bf16 MFMA expert-FFN kernels for gfx950 (MI355X): grouped GEMMs over variable-length expert
-// segments with the SwiGLU forward / backward fused into the epilogues.
+// segments, forward + dgrad + wgrad, with the SwiGLU forward / backward fused into the epilogues.
 //
 // Block tile 256 x 256 x 64 (M x N x K), 4 wavefronts (one per SIMD), each owning a 128 x 128
-// sub-tile as 4 x 4 v_mfma_f32_32x32x16_bf16 accumulators (256 fp32 per lane).  Operand tiles go
-// HBM -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of 64 KB.
-// LDS rows are 128 B (64 bf16 of K); the 16-byte chunk index is XOR-swizzled with the row so the
-// ds_read_b128 fragment reads of 32 consecutive rows spread over all banks.  The swizzle is applied
-// on the global-address side because a direct-to-LDS load always writes lane l at LDS base + 16*l.
+// sub-tile as 4 x 4 v_mfma_f32_32x32x16_bf16 accumulators (256 fp32 per lane, in AGPRs).  Operand
+// tiles go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of
+// 64 KB; a stage is refilled right after the barrier that frees it, half of the loads there and half
+// one k-sub-step later, interleaved with MFMAs so the in-order wave never blocks on the memory queue.
+//
+// Two LDS tile layouts, chosen per operand by how it lies in memory:
+//   K-major  (rows of the operand are contiguous along K: activations, forward weights)
+//            LDS [256 rows][64 k] (128 B rows); fragments are plain ds_read_b128; the 16-byte chunk index
+//            is XOR-swizzled with the row.
+//   X-major  (contiguous along M or N, i.e. K is the slow index: weights in dgrad, both operands of wgrad)
+//            LDS [64 k][256 cols] (512 B rows); fragments come from ds_read_b64_tr_b16, the LDS
+//            transpose-read of gfx950, so no transposed copy of any tensor is ever made.
+// A direct-to-LDS load always writes lane l at LDS base + 16*l, so every swizzle is applied on the
+// global-address side (which 16-byte chunk a lane fetches).
 //
 // Tiles are enumerated on the device from counts[] (no host copy): expert by expert, N-tile by
 // N-tile, M-tile fastest, and consecutive tiles are handed to the same XCD (block b runs on XCD
-// b % 8) so that the blocks sharing an L2 share weight tiles.
+// b % 8) so that the blocks sharing an L2 share operand tiles.
 #include "ffn.h"
 
 namespace {
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kTileBytesA = BM * BK * 2;  // 32 KB
-constexpr int kTileBytesB = BN * BK * 2;  // 32 KB
-constexpr int kStageBytes = kTileBytesA + kTileBytesB;
+constexpr int kTileBytes = 256 * BK * 2;  // 32 KB per operand tile
+constexpr int kStageBytes = 2 * kTileBytes;
 constexpr int kNumXcd = 8;
 
-enum Mode { kGateUp = 0, kDown = 1 };
+enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
+
+template <int MODE>
+struct Traits {
+    static constexpr bool kAKMajor = MODE != kWgrad;
+    static constexpr bool kBKMajor = MODE == kGateUp || MODE == kDown;
+};
 
 struct MfmaParams {
     const int64_t* counts;
     int E;
     int64_t n_rows;
-    int64_t K;         // contraction length (H for gate/up, I for down)
-    int64_t n_cols;    // output columns the N tiles cover (I for gate/up: 128 per tile; H for down: 256 per tile)
-    int n_tiles;
-    const uint16_t* A;   // [n_rows, K]
-    const uint16_t* B0;  // gate_w [E, I, H] or down_w [E, H, I]
+    int64_t K;          // contraction length for the M-grouped modes
+    int64_t N;          // output columns (I for gate/up and dgrad_act, H for down and dgrad_x, Q for wgrad)
+    int64_t M;          // wgrad only: output rows P
+    int n_tiles;        // tiles along N
+    int m_tiles;        // wgrad only: tiles along P
+    const uint16_t* A;  // activations [n_rows, lda]; wgrad: lhs
+    int64_t lda;
+    const uint16_t* B0;  // gate_w / down_w; wgrad: rhs
     const uint16_t* B1;  // up_w or null
-    uint16_t* out;       // act [n_rows, I] or y [n_rows, H]
-    uint16_t* inter13;   // optional [n_rows, 2I]
-    const uint16_t* row_weight;
+    int64_t ldb;         // row stride of B (elements)
+    int64_t b_expert_stride;
+    uint16_t* out;
+    int64_t ldo;
+    uint16_t* out2;       // gate/up: inter13 (optional); dgrad_act: act_out (optional)
+    const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
 };
 
 __device__ __forceinline__ int swz(int row) { return (row + (row >> 3)) & 7; }
+// X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
+__device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
 
 __device__ __forceinline__ void load16_to_lds(const void* g, char* l) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
                                      (__attribute__((address_space(3))) void*)l, 16, 0, 0);
 }
 
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+__device__ __forceinline__ s16x4_t lds_read_tr(const char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
+}
+
 struct TileCoord {
-    int e, n_tile, rows;
-    int64_t row0;
+    int e, n_tile, m_tile, rows;  // rows: valid M rows (M-grouped) or valid K rows (wgrad)
+    int64_t row0;                 // first row of the tile (M-grouped) or of the expert segment (wgrad)
 };
 
-// Logical tile id -> (expert, N tile, M tile).  Returns false for ids past the last tile.
-__device__ __forceinline__ bool locate(const int64_t* counts, int E, int n_tiles, TileCoord* tc) {
-    int64_t total_m = 0;
-    for (int e = 0; e < E; ++e) total_m += (counts[e] + BM - 1) / BM;
-    const int64_t total = total_m * n_tiles;
+// Logical tile id of this block with the XCD remap, or -1.
+__device__ __forceinline__ int64_t logical_tile(int64_t total) {
     const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
     const int64_t slot = blockIdx.x / kNumXcd;
-    if (slot >= per_xcd) return false;
-    int64_t L = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
-    if (L >= total) return false;
+    if (slot >= per_xcd) return -1;
+    const int64_t L = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
+    return L < total ? L : -1;
+}
+
+__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, TileCoord* tc) {
+    int64_t total_m = 0;
+    for (int e = 0; e < E; ++e) total_m += (counts[e] + BM - 1) / BM;
+    int64_t L = logical_tile(total_m * n_tiles);
+    if (L < 0) return false;
     int64_t start = 0;
     for (int e = 0; e < E; ++e) {
         const int64_t c = counts[e];
@@ -68,6 +100,7 @@ __device__ __forceinline__ bool locate(const int64_t* counts, int E, int n_tiles
         if (L < te) {
             const int m = (int)(L % me);
             tc->e = e;
+            tc->m_tile = m;
             tc->n_tile = (int)(L / me);
             tc->row0 = start + (int64_t)m * BM;
             const int64_t left = c - (int64_t)m * BM;
@@ -80,56 +113,152 @@ __device__ __forceinline__ bool locate(const int64_t* counts, int E, int n_tiles
     return false;
 }
 
+__device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, TileCoord* tc) {
+    const int64_t per_e = (int64_t)m_tiles * n_tiles;
+    const int64_t L = logical_tile(per_e * E);
+    if (L < 0) return false;
+    const int e = (int)(L / per_e);
+    const int64_t rem = L % per_e;
+    tc->e = e;
+    tc->n_tile = (int)(rem / m_tiles);
+    tc->m_tile = (int)(rem % m_tiles);
+    int64_t start = 0;
+    for (int i = 0; i < e; ++i) start += counts[i];
+    tc->row0 = start;
+    tc->rows = (int)counts[e];
+    return true;
+}
+
 template <int MODE>
-__global__ __launch_bounds__(256, 1) void ffn_mfma_tn_kernel(MfmaParams p) {
+__global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
+    using T = Traits<MODE>;
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
-    if (!locate(p.counts, p.E, p.n_tiles, &tc)) return;
+    if (MODE == kWgrad) {
+        if (!locate_wgrad(p.counts, p.E, p.m_tiles, p.n_tiles, &tc)) return;
+    } else {
+        if (!locate_m_grouped(p.counts, p.E, p.n_tiles, &tc)) return;
+    }
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t K = p.K;
+    const int l31 = lane & 31, hi = lane >> 5;
+    const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
 
-    // ---- global -> LDS assignment: wave w fills tile rows [64w, 64w+64) of A and of B, 8 rows per instruction
-    const int lrow = lane >> 3, lchunk = lane & 7;
+    // ------------------------------------------------------------------------------------------
+    // global -> LDS: per lane, the source of each of the wave's 8 load instructions per operand
+    // ------------------------------------------------------------------------------------------
     const char* a_src[8];
     const char* b_src[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-        const int r = wave * 64 + q * 8 + lrow;
-        const int gchunk = lchunk ^ swz(r);
-        const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the expert's last one re-read it (never stored)
-        a_src[q] = (const char*)(p.A + (tc.row0 + ar) * K) + gchunk * 16;
-        int64_t brow;
-        const uint16_t* bmat;
-        if (MODE == kGateUp) {
-            bmat = ((r & 127) < 64) ? p.B0 : p.B1;
-            brow = (int64_t)tc.e * p.n_cols + (int64_t)tc.n_tile * 128 + (r >> 7) * 64 + (r & 63);
-        } else {
-            bmat = p.B0;
-            brow = (int64_t)tc.e * p.n_cols + (int64_t)tc.n_tile * BN + r;
-        }
-        b_src[q] = (const char*)(bmat + brow * K) + gchunk * 16;
-    }
-    auto issue_loads = [&](int kt, int stage) {
-        char* base = lds + stage * kStageBytes + (wave * 64) * 128;
+    int64_t a_step, b_step;      // bytes per k-tile
+    int64_t b_switch_delta = 0;  // dgrad_x: jump from gate_w to up_w half way through K
+    int b_switch_kt = 0x7FFFFFFF;
+    if (T::kAKMajor) {
+        // wave w fills tile rows [64w, 64w+64), 8 rows (128 B each) per instruction
+        a_step = BK * 2;
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            load16_to_lds(a_src[q] + (int64_t)kt * (BK * 2), base + q * 1024);
-            load16_to_lds(b_src[q] + (int64_t)kt * (BK * 2), base + kTileBytesA + q * 1024);
+            const int r = wave * 64 + q * 8 + (lane >> 3);
+            const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the segment re-read its last row (never stored)
+            a_src[q] = (const char*)(p.A + (tc.row0 + ar) * p.lda) + ((lane & 7) ^ swz(r)) * 16;
+        }
+    } else {
+        // wgrad lhs [k rows, P]: wave w fills k rows [16w, 16w+16), 2 rows (512 B each) per instruction
+        a_step = BK * p.lda * 2;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int kr = wave * 16 + q * 2 + (lane >> 5);
+            const int chunk = (lane & 31) ^ swz_x(kr);
+            int64_t col = (int64_t)tc.m_tile * BM + chunk * 8;
+            col = col + 8 <= p.M ? col : p.M - 8;
+            a_src[q] = (const char*)(p.A + (tc.row0 + kr) * p.lda + col);
+        }
+    }
+    if (T::kBKMajor) {
+        b_step = BK * 2;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int r = wave * 64 + q * 8 + (lane >> 3);
+            int64_t brow;
+            const uint16_t* bmat;
+            if (MODE == kGateUp) {
+                // B tile rows: per wave column, 64 gate rows then 64 up rows of the same I range
+                bmat = ((r & 127) < 64) ? p.B0 : p.B1;
+                brow = (int64_t)tc.n_tile * 128 + (r >> 7) * 64 + (r & 63);
+            } else {
+                bmat = p.B0;
+                brow = (int64_t)tc.n_tile * BN + r;
+            }
+            b_src[q] = (const char*)(bmat + (int64_t)tc.e * p.b_expert_stride + brow * p.ldb) + ((lane & 7) ^ swz(r)) * 16;
+        }
+    } else {
+        b_step = BK * p.ldb * 2;
+        const uint16_t* bmat = MODE == kWgrad ? p.B0 + tc.row0 * p.ldb : p.B0 + (int64_t)tc.e * p.b_expert_stride;
+        if (MODE == kDgradX) {
+            b_switch_kt = n_kt / 2;
+            b_switch_delta = ((const char*)p.B1 - (const char*)p.B0) - (int64_t)b_switch_kt * b_step;
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int kr = wave * 16 + q * 2 + (lane >> 5);
+            const int chunk = (lane & 31) ^ swz_x(kr);
+            int64_t col = (int64_t)tc.n_tile * BN + chunk * 8;
+            col = col + 8 <= p.N ? col : p.N - 8;
+            b_src[q] = (const char*)(bmat + (int64_t)kr * p.ldb + col);
+        }
+    }
+    // wgrad: k rows past the expert's last row are re-read from its last row and masked out of the fragments
+    auto k_clamp = [&](int kt, int q) -> int64_t {
+        if (MODE != kWgrad) return 0;
+        const int kr = kt * BK + wave * 16 + q * 2 + (lane >> 5);
+        return kr < tc.rows ? 0 : (int64_t)(tc.rows - 1 - kr);
+    };
+    auto issue_loads_part = [&](int kt, int stage, int q0) {
+        char* base = lds + stage * kStageBytes;
+        const int64_t b_off = (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
+#pragma unroll
+        for (int q = q0; q < q0 + 4; ++q) {
+            const int64_t dk = k_clamp(kt, q);
+            if (T::kAKMajor)
+                load16_to_lds(a_src[q] + (int64_t)kt * a_step, base + (wave * 64 + q * 8) * 128);
+            else
+                load16_to_lds(a_src[q] + (int64_t)kt * a_step + dk * p.lda * 2, base + (wave * 16 + q * 2) * 512);
+            if (T::kBKMajor)
+                load16_to_lds(b_src[q] + b_off, base + kTileBytes + (wave * 64 + q * 8) * 128);
+            else
+                load16_to_lds(b_src[q] + b_off + dk * p.ldb * 2, base + kTileBytes + (wave * 16 + q * 2) * 512);
         }
     };
 
-    // ---- fragment addressing: lane reads row (l & 31) of a 32-row block, k chunk (2*kk + (l >> 5))
-    const int l31 = lane & 31, hi = lane >> 5;
+    // ------------------------------------------------------------------------------------------
+    // LDS -> fragments
+    // ------------------------------------------------------------------------------------------
+    // K-major: lane reads row (l & 31) of a 32-row block, 16-byte k chunk (2*kk + (l >> 5)).
+    // X-major: two transpose reads per fragment; lane addresses 8 bytes of k row 16kk + 8*(l>>5) + 4t + ((l>>2)&3)
+    //          at column 16*((l>>4)&1) + 4*(l&3) of the 32-column block and receives k rows 16kk + 8*(l>>5) + 4t..+3
+    //          of column 16*((l>>4)&1) + (l&15).
     int a_rd[4], b_rd[4], a_f[4], b_f[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int ra = wm * 128 + i * 32 + l31, rb = wn * 128 + i * 32 + l31;
-        a_rd[i] = ra * 128;
-        a_f[i] = swz(ra);
-        b_rd[i] = kTileBytesA + rb * 128;
-        b_f[i] = swz(rb);
+        const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
+        if (T::kAKMajor) {
+            const int ra = wm * 128 + i * 32 + l31;
+            a_rd[i] = ra * 128;
+            a_f[i] = swz(ra);
+        } else {
+            const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            a_rd[i] = (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            a_f[i] = 0;
+        }
+        if (T::kBKMajor) {
+            const int rb = wn * 128 + i * 32 + l31;
+            b_rd[i] = kTileBytes + rb * 128;
+            b_f[i] = swz(rb);
+        } else {
+            const int col = wn * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            b_rd[i] = kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            b_f[i] = 0;
+        }
     }
 
     f32x16_t acc[4][4];
@@ -141,12 +270,44 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_tn_kernel(MfmaParams p) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     bf16x8_t af[2][4], bfr[2][4];
+    auto read_tr_frag = [&](const char* base, int kk) -> bf16x8_t {
+        const s16x4_t lo = lds_read_tr(base + kk * (16 * 512));
+        const s16x4_t hi4 = lds_read_tr(base + kk * (16 * 512) + 4 * 512);
+        const s16x8_t v = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        return __builtin_bit_cast(bf16x8_t, v);
+    };
     auto read_frags = [&](int stage, int kk, int buf) {
         const char* sb = lds + stage * kStageBytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            af[buf][i] = *(const bf16x8_t*)(sb + a_rd[i] + (((kk * 2 + hi) ^ a_f[i]) << 4));
-            bfr[buf][i] = *(const bf16x8_t*)(sb + b_rd[i] + (((kk * 2 + hi) ^ b_f[i]) << 4));
+            if (T::kAKMajor)
+                af[buf][i] = *(const bf16x8_t*)(sb + a_rd[i] + (((kk * 2 + hi) ^ a_f[i]) << 4));
+            else
+                af[buf][i] = read_tr_frag(sb + a_rd[i], kk);
+            if (T::kBKMajor)
+                bfr[buf][i] = *(const bf16x8_t*)(sb + b_rd[i] + (((kk * 2 + hi) ^ b_f[i]) << 4));
+            else
+                bfr[buf][i] = read_tr_frag(sb + b_rd[i], kk);
+        }
+    };
+    // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
+    auto mask_tail = [&](int kt, int kk, int buf) {
+        if (MODE != kWgrad) return;
+        const int valid = tc.rows - kt * BK - kk * 16 - 8 * hi;  // lane holds k = 8*hi + 0..7 of this sub-step
+        if (valid >= 8) return;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s16x8_t a = __builtin_bit_cast(s16x8_t, af[buf][i]);
+            s16x8_t b = __builtin_bit_cast(s16x8_t, bfr[buf][i]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (e >= valid) {
+                    a[e] = 0;
+                    b[e] = 0;
+                }
+            }
+            af[buf][i] = __builtin_bit_cast(bf16x8_t, a);
+            bfr[buf][i] = __builtin_bit_cast(bf16x8_t, b);
         }
     };
     auto mma = [&](int buf) {
@@ -157,79 +318,187 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_tn_kernel(MfmaParams p) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
     };
 
-    const int n_kt = (int)(K / BK);
-    issue_loads(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    read_frags(0, 0, 0);
-    for (int kt = 0; kt < n_kt; ++kt) {
-        const int stage = kt & 1;
-        if (kt + 1 < n_kt) issue_loads(kt + 1, stage ^ 1);
-        read_frags(stage, 1, 1);
-        mma(0);
-        read_frags(stage, 2, 0);
-        mma(1);
-        read_frags(stage, 3, 1);
-        mma(0);
-        // every wave has read its last fragments of this stage; the next tile must have landed
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        if (kt + 1 < n_kt) read_frags(stage ^ 1, 0, 0);
-        mma(1);
+    // One k-sub-step = the fragment reads of the NEXT sub-step (and, in two of the four sub-steps, half of the
+    // direct-to-LDS loads of a later tile) interleaved with the 16 MFMAs of this sub-step.
+    constexpr int kReadsPerGroup = ((T::kAKMajor ? 4 : 8) + (T::kBKMajor ? 4 : 8)) / 8;
+#define PICOMOE_INTERLEAVE(WITH_LOADS)                                            \
+    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                            \
+        __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerGroup, 0);           \
+        if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                        \
     }
 
-    // ---- epilogue: lane holds column (l & 31), rows 8*(r/4) + 4*(l >> 5) + (r % 4) of each 32 x 32 block
+    if (n_kt > 0) {
+        issue_loads_part(0, 0, 0);
+        issue_loads_part(0, 0, 4);
+        if (n_kt > 1) {
+            issue_loads_part(1, 1, 0);
+            issue_loads_part(1, 1, 4);
+            __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 landed, tile 1 may still be in flight
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();
+        read_frags(0, 0, 0);
+    }
+    for (int kt = 0; kt < n_kt; ++kt) {
+        const int stage = kt & 1;
+        const bool tail = MODE == kWgrad && kt == n_kt - 1;
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt > 0 && kt + 1 < n_kt) issue_loads_part(kt + 1, stage ^ 1, 4);  // second half of the refill begun last step
+        if (tail) mask_tail(kt, 0, 0);
+        read_frags(stage, 1, 1);
+        mma(0);
+        PICOMOE_INTERLEAVE(true)
+        __builtin_amdgcn_sched_barrier(0);
+        if (tail) mask_tail(kt, 1, 1);
+        read_frags(stage, 2, 0);
+        mma(1);
+        PICOMOE_INTERLEAVE(false)
+        __builtin_amdgcn_sched_barrier(0);
+        if (tail) mask_tail(kt, 2, 0);
+        read_frags(stage, 3, 1);
+        mma(0);
+        PICOMOE_INTERLEAVE(false)
+        __builtin_amdgcn_sched_barrier(0);
+        // Every wave holds its last fragments of this stage in registers and the next tile has landed:
+        // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        if (kt + 2 < n_kt) issue_loads_part(kt + 2, stage, 0);
+        if (tail) mask_tail(kt, 3, 1);
+        if (kt + 1 < n_kt) read_frags(stage ^ 1, 0, 0);
+        mma(1);
+        PICOMOE_INTERLEAVE(true)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#undef PICOMOE_INTERLEAVE
+
+    // ------------------------------------------------------------------------------------------
+    // epilogue.  A lane holds column (l & 31) and rows 8*(r/4) + 4*(l >> 5) + (r % 4) of each 32 x 32
+    // accumulator block: consecutive lanes are consecutive columns, 2 bytes apart in the output.  Each wave
+    // therefore stages 32 rows at a time through its own slice of LDS (the operand stages are free after
+    // the last barrier) and reads them back row-contiguously, so HBM sees 16-byte lanes and 128..256-byte
+    // row segments, and the fused SwiGLU backward reads g / u the same way.
+    // ------------------------------------------------------------------------------------------
+    int valid_rows = tc.rows;
+    int64_t out_row0 = tc.row0;
+    if (MODE == kWgrad) {
+        const int64_t left = p.M - (int64_t)tc.m_tile * BM;
+        valid_rows = left < BM ? (int)left : BM;
+        out_row0 = (int64_t)tc.e * p.M + (int64_t)tc.m_tile * BM;
+    }
+    constexpr int kEpiCols = MODE == kGateUp ? 64 : 128;  // output columns per wave and pass
+    constexpr int kEpiStride = (kEpiCols + 8) * 2;        // bytes; the 16-byte pad rotates rows over the banks
+    char* epi = lds + wave * (32 * kEpiStride);
+    constexpr int kChunksPerRow = kEpiCols / 8;
+    constexpr int kReadIters = 32 * kChunksPerRow / 64;
+
+    auto stage_block = [&](auto value) {  // value(j, r) -> float, j over the 32-column blocks of this pass
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // earlier read-backs of this slice are done
+#pragma unroll
+        for (int j = 0; j < kEpiCols / 32; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
+                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + l31) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    // for_chunks(i, f): f(row_in_tile, col_in_wave_pass, 8 staged bf16 as u32x4)
+    auto for_chunks = [&](int i, auto f) {
+#pragma unroll
+        for (int it = 0; it < kReadIters; ++it) {
+            const int idx = it * 64 + lane;
+            const int row = idx / kChunksPerRow, ch = idx % kChunksPerRow;
+            const u32x4_t v = *(const u32x4_t*)(epi + row * kEpiStride + ch * 16);
+            const int trow = wm * 128 + i * 32 + row;
+            if (trow < valid_rows) f(trow, ch * 8, v);
+        }
+    };
+
     if (MODE == kGateUp) {
-        const int64_t I = p.n_cols;
+        const int64_t I = p.N;
+        const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * 64;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            // g and u rounded to bf16 in place (what the reference's two Linear outputs hold)
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const int64_t col = (int64_t)tc.n_tile * 128 + wn * 64 + jj * 32 + l31;
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-                    if (row < tc.rows) {
-                        const float g = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][jj][r]));
-                        const float u = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][jj + 2][r]));
-                        const float s = bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g)));
-                        const int64_t grow = tc.row0 + row;
-                        p.out[grow * I + col] = (uint16_t)f32_to_bf16_bits(s * u);
-                        if (p.inter13) {
-                            p.inter13[grow * 2 * I + col] = (uint16_t)f32_to_bf16_bits(g);
-                            p.inter13[grow * 2 * I + I + col] = (uint16_t)f32_to_bf16_bits(u);
-                        }
-                    }
-                }
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][r]));
+            stage_block([&](int j, int r) {
+                const float g = acc[i][j][r], u = acc[i][j + 2][r];
+                return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
+            });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v; });
+            if (p.out2) {
+                stage_block([&](int j, int r) { return acc[i][j][r]; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v; });
+                stage_block([&](int j, int r) { return acc[i][j + 2][r]; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v; });
             }
         }
     } else {
-        const int64_t H = p.n_cols;
+        const int64_t col0 = (int64_t)tc.n_tile * BN + wn * 128;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            stage_block([&](int j, int r) { return acc[i][j][r]; });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) {
+                const int64_t col = col0 + c;
+                if (col >= p.N) return;
+                const int64_t grow = out_row0 + trow;
+                if (MODE == kDgradAct) {
+                    const int64_t I = p.N;
+                    const u32x4_t gv = *(const u32x4_t*)(p.aux + grow * 2 * I + col);
+                    const u32x4_t uv = *(const u32x4_t*)(p.aux + grow * 2 * I + I + col);
+                    u32x4_t dgv, duv, av;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t col = (int64_t)tc.n_tile * BN + wn * 128 + j * 32 + l31;
+                    for (int w2 = 0; w2 < 4; ++w2) {
+                        float o_dg[2], o_du[2], o_a[2];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-                    if (row < tc.rows) {
-                        const int64_t grow = tc.row0 + row;
-                        float v = acc[i][j][r];
-                        if (p.row_weight)
-                            v = bf16_bits_to_f32(f32_to_bf16_bits(v)) * bf16_bits_to_f32(p.row_weight[grow]);
-                        p.out[grow * H + col] = (uint16_t)f32_to_bf16_bits(v);
+                        for (int h2 = 0; h2 < 2; ++h2) {
+                            const float da = __uint_as_float(h2 ? (v[w2] & 0xFFFF0000u) : (v[w2] << 16));
+                            const float g = __uint_as_float(h2 ? (gv[w2] & 0xFFFF0000u) : (gv[w2] << 16));
+                            const float u = __uint_as_float(h2 ? (uv[w2] & 0xFFFF0000u) : (uv[w2] << 16));
+                            const float sig = sigmoid_fast(g);
+                            o_dg[h2] = da * u * (sig * (1.f + g * (1.f - sig)));
+                            o_du[h2] = da * (g * sig);
+                            o_a[h2] = bf16_bits_to_f32(f32_to_bf16_bits(g * sig)) * u;
+                        }
+                        dgv[w2] = pack_bf16x2(o_dg[0], o_dg[1]);
+                        duv[w2] = pack_bf16x2(o_du[0], o_du[1]);
+                        av[w2] = pack_bf16x2(o_a[0], o_a[1]);
                     }
+                    *(u32x4_t*)(p.out + grow * 2 * I + col) = dgv;
+                    *(u32x4_t*)(p.out + grow * 2 * I + I + col) = duv;
+                    if (p.out2) *(u32x4_t*)(p.out2 + grow * I + col) = av;
+                } else if (MODE == kDown && p.aux) {
+                    const float rw = bf16_bits_to_f32(p.aux[grow]);
+                    u32x4_t o;
+#pragma unroll
+                    for (int w2 = 0; w2 < 4; ++w2)
+                        o[w2] = pack_bf16x2(__uint_as_float(v[w2] << 16) * rw, __uint_as_float(v[w2] & 0xFFFF0000u) * rw);
+                    *(u32x4_t*)(p.out + grow * p.ldo + col) = o;
+                } else {
+                    *(u32x4_t*)(p.out + grow * p.ldo + col) = v;
                 }
-            }
+            });
         }
     }
 }
 
-inline unsigned grid_bound(const FfnShape& s, int n_tiles) {
-    const int64_t m_bound = s.n_rows / BM + s.E;
-    const int64_t g = m_bound * n_tiles;
-    return (unsigned)(((g + kNumXcd - 1) / kNumXcd) * kNumXcd);
+inline unsigned round_up_xcd(int64_t g) { return (unsigned)(((g + kNumXcd - 1) / kNumXcd) * kNumXcd); }
+inline unsigned grid_m_grouped(const FfnShape& s, int n_tiles) {
+    return round_up_xcd((s.n_rows / BM + s.E) * (int64_t)n_tiles);
+}
+
+MfmaParams base_params(const FfnShape& s) {
+    MfmaParams p{};
+    p.counts = s.counts;
+    p.E = s.E;
+    p.n_rows = s.n_rows;
+    return p;
 }
 
 }  // namespace
@@ -240,33 +509,61 @@ bool ffn_mfma_supported(const FfnShape& s) {
 
 int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
                      hipStream_t st) {
-    MfmaParams p{};
-    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.K = s.H; p.n_cols = s.I; p.n_tiles = (int)(s.I / 128);
-    p.A = (const uint16_t*)x; p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w;
-    p.out = (uint16_t*)act; p.inter13 = (uint16_t*)inter13; p.row_weight = nullptr;
-    hipLaunchKernelGGL(ffn_mfma_tn_kernel<kGateUp>, dim3(grid_bound(s, p.n_tiles)), dim3(256), 0, st, p);
+    MfmaParams p = base_params(s);
+    p.K = s.H; p.N = s.I; p.n_tiles = (int)(s.I / 128);
+    p.A = (const uint16_t*)x; p.lda = s.H;
+    p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;
+    p.out = (uint16_t*)act; p.ldo = s.I; p.out2 = (uint16_t*)inter13;
+    hipLaunchKernelGGL(ffn_mfma_kernel<kGateUp>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
 int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, hipStream_t st) {
-    MfmaParams p{};
-    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.K = s.I; p.n_cols = s.H; p.n_tiles = (int)(s.H / BN);
-    p.A = (const uint16_t*)act; p.B0 = (const uint16_t*)down_w; p.B1 = nullptr;
-    p.out = (uint16_t*)y; p.inter13 = nullptr; p.row_weight = (const uint16_t*)row_weight;
-    hipLaunchKernelGGL(ffn_mfma_tn_kernel<kDown>, dim3(grid_bound(s, p.n_tiles)), dim3(256), 0, st, p);
+    MfmaParams p = base_params(s);
+    p.K = s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
+    p.A = (const uint16_t*)act; p.lda = s.I;
+    p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;
+    p.out = (uint16_t*)y; p.ldo = s.H; p.aux = (const uint16_t*)row_weight;
+    hipLaunchKernelGGL(ffn_mfma_kernel<kDown>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
-// The backward GEMMs still run on the generic kernels.
 int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, const void* inter13, void* d_inter13,
                        void* act_out, hipStream_t st) {
-    return ffn_simple_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, st);
+    MfmaParams p = base_params(s);
+    p.K = s.H; p.N = s.I; p.n_tiles = (int)((s.I + BN - 1) / BN);
+    p.A = (const uint16_t*)dy; p.lda = s.H;
+    p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;  // down_w[e] read as [K = H][N = I]
+    p.out = (uint16_t*)d_inter13; p.ldo = 2 * s.I; p.out2 = (uint16_t*)act_out; p.aux = (const uint16_t*)inter13;
+    hipLaunchKernelGGL(ffn_mfma_kernel<kDgradAct>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    return picomoe_launch_status();
 }
+
 int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx,
                      hipStream_t st) {
-    return ffn_simple_dgrad_x(s, d_inter13, gate_w, up_w, dx, st);
+    MfmaParams p = base_params(s);
+    p.K = 2 * s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
+    p.A = (const uint16_t*)d_inter13; p.lda = 2 * s.I;
+    p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;  // [K = I][N = H]
+    p.out = (uint16_t*)dx; p.ldo = s.H;
+    hipLaunchKernelGGL(ffn_mfma_kernel<kDgradX>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    return picomoe_launch_status();
 }
+
+bool ffn_mfma_wgrad_supported(int dtype, int64_t P, int64_t Q, int64_t ld_lhs, int64_t ld_rhs, const void* lhs,
+                              const void* rhs) {
+    return dtype == PICOMOE_BF16 && P % 8 == 0 && Q % 8 == 0 && P >= 128 && Q >= 128 && ld_lhs % 8 == 0 &&
+           ld_rhs % 8 == 0 && (uintptr_t)lhs % 16 == 0 && (uintptr_t)rhs % 16 == 0;
+}
+
 int ffn_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, int64_t P, int64_t Q,
                    void* out, hipStream_t st) {
-    return ffn_simple_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, P, Q, out, st);
+    MfmaParams p = base_params(s);
+    p.M = P; p.N = Q; p.m_tiles = (int)((P + BM - 1) / BM); p.n_tiles = (int)((Q + BN - 1) / BN);
+    p.A = (const uint16_t*)lhs; p.lda = ld_lhs;
+    p.B0 = (const uint16_t*)rhs; p.ldb = ld_rhs;
+    p.out = (uint16_t*)out; p.ldo = Q;
+    const int64_t tiles = (int64_t)s.E * p.m_tiles * p.n_tiles;
+    hipLaunchKernelGGL(ffn_mfma_kernel<kWgrad>, dim3(round_up_xcd(tiles)), dim3(256), 0, st, p);
+    return picomoe_launch_status();
 }
