@@ -1,0 +1,304 @@
+#!/usr/bin/env python3
+"""Benchmark of the single-GPU MoE hot path on MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c4]
+
+A "step" is one pass of the hot path over one batch of synthetic input.  The default workload is the
+Mixtral-shape MoE layer forward + backward with FP8 dispatch (8192 tokens, hidden 4096, FFN 14336, 8 experts,
+top-2, bf16, aux-loss coefficient 0.01): zero_grad, forward, loss = <out, g> + aux, backward -- every gradient
+the reference's autograd produces (input, router, 3 x 8 expert matrices) is computed inside the timed region.
+Inputs and weights are resident in HBM before the clock starts.
+
+Prints ONE JSON line on stdout: the layer's tokens/s as `value`, a `roofline` object for the grouped-GEMM
+kernels (algorithmic FLOP / launch durations measured here with events on the launch stream), the FP8
+quantise bandwidth and a `cpu_baseline` (the CPU oracle timed on this box's host cores on a bounded sample).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+import types
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+WORKLOADS = {
+    # name: tokens, hidden, ffn, experts, top_k, shared, capacity_factor, fp8_dispatch, backward
+    "c5": dict(T=8192, H=4096, I=14336, E=8, k=2, shared=0, cap=0.0, fp8=True, bwd=True,
+               desc="Mixtral-shape MoE layer fwd+bwd, FP8 dispatch, aux 0.01: 8192 tok, H4096, I14336, E8, top-2, bf16"),
+    "c3": dict(T=8192, H=4096, I=14336, E=8, k=2, shared=0, cap=0.0, fp8=False, bwd=False,
+               desc="Mixtral-shape MoE layer fwd: 8192 tok, H4096, I14336, E8, top-2, bf16"),
+    "c4": dict(T=16384, H=2048, I=1408, E=64, k=6, shared=2, cap=1.25, fp8=False, bwd=False,
+               desc="fine-grained skewed MoE fwd: 16384 tok, H2048, I1408, E64, top-6, shared 2816, capacity 1.25 drop"),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_layer(w, device, dtype):
+    import torch
+
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer
+
+    cfg = types.SimpleNamespace(
+        hidden_size=w["H"], intermediate_size=w["I"], num_experts=w["E"], num_experts_per_tok=w["k"],
+        num_shared_experts=w["shared"], norm_topk_prob=True, ep_fp8_dispatch=w["fp8"],
+        ep_capacity_factor=w["cap"], ep_capacity_dropless=False, router_aux_loss_coef=0.01 if w["bwd"] else 0.0,
+    )
+    with torch.device("meta"):
+        moe = MoELayer(cfg)
+    moe = moe.to_empty(device=device).to(dtype)
+    g = torch.Generator(device=device).manual_seed(0)
+    with torch.no_grad():
+        for p in moe.parameters():
+            p.copy_((0.02 * torch.randn(p.shape, generator=g, device=device, dtype=torch.float32)).to(dtype))
+        moe.expert_bias.zero_()
+        if w["cap"] > 0:  # Zipf(s=1.1) router bias -> load imbalance
+            moe.gate.bias = torch.nn.Parameter(
+                (-1.1 * torch.log(torch.arange(1, w["E"] + 1, device=device, dtype=torch.float32))).to(dtype))
+    moe.train(w["bwd"])
+    return moe
+
+
+def time_events(fn, iters, warm=2):
+    import torch
+
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    st.record()
+    for _ in range(iters):
+        fn()
+    en.record()
+    torch.cuda.synchronize()
+    return st.elapsed_time(en) / iters  # ms
+
+
+class GemmTimer:
+    """Records an event pair on the launch stream around every grouped-GEMM launch of the timed steps, so the
+    launch durations come from the same region the throughput figure does."""
+
+    FLOP = {"gate_up": 4.0, "down": 2.0, "dgrad_act": 2.0, "dgrad_x": 4.0, "wgrad": 2.0}  # x routed rows x H x I
+
+    def __init__(self):
+        self.records = []
+        self.enabled = False
+
+    def install(self):
+        import torch
+
+        from picotron_amd.expert_parallel import megakernel as mk
+
+        def wrap(name, fn):
+            def timed(*a, **kw):
+                if not self.enabled:
+                    return fn(*a, **kw)
+                st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                st.record()
+                out = fn(*a, **kw)
+                en.record()
+                label = name
+                if name == "wgrad":  # (lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset)
+                    label = "wgrad_down" if a[1] == a[7] else ("wgrad_up" if kw.get("lhs_offset", 0) else "wgrad_gate")
+                self.records.append((label, name, st, en))
+                return out
+            return timed
+
+        for name in ("gate_up", "down", "dgrad_act", "dgrad_x", "wgrad"):
+            setattr(mk, "_" + name, wrap(name, getattr(mk, "_" + name)))
+
+    def summary(self, routed_rows, H, I):
+        per = {}
+        for label, name, st, en in self.records:
+            d = per.setdefault(label, {"ms": 0.0, "n": 0, "flop": self.FLOP[name] * routed_rows * H * I})
+            d["ms"] += st.elapsed_time(en)
+            d["n"] += 1
+        return {k: (v["ms"] / v["n"], v["flop"], v["n"]) for k, v in per.items()}
+
+
+def fp8_quant_bandwidth(device, n=16384, h=4096, sets=6, iters=60):
+    """FP8 E4M3 dispatch quantise at 16384 x 4096 bf16, rotating over buffer sets larger than the 256 MB
+    last-level cache so the figure is HBM traffic.  Returns (GB/s quantise, GB/s dequantise)."""
+    import torch
+
+    from picotron_amd import _lib
+
+    lib = _lib.load()
+    xs = [torch.randn(n, h, device=device).bfloat16() for _ in range(sets)]
+    qs = [torch.empty(n, h, dtype=torch.uint8, device=device) for _ in range(sets)]
+    ss = [torch.empty(n, dtype=torch.float32, device=device) for _ in range(sets)]
+    os_ = [torch.empty(n, h, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    st = _lib.stream_ptr()
+    state = {"i": 0}
+
+    def quant():
+        i = state["i"] = (state["i"] + 1) % sets
+        lib.picomoe_fp8_quant(_lib.ptr(xs[i]), 1, n, h, _lib.ptr(qs[i]), _lib.ptr(ss[i]), st)
+
+    def dequant():
+        i = state["i"] = (state["i"] + 1) % sets
+        lib.picomoe_fp8_dequant(_lib.ptr(qs[i]), _lib.ptr(ss[i]), n, h, _lib.ptr(os_[i]), 1, st)
+
+    nbytes = n * h * 3 + n * 4
+    tq = time_events(quant, iters, warm=sets)
+    td = time_events(dequant, iters, warm=sets)
+    return nbytes / tq / 1e6, nbytes / td / 1e6, tq * 1e3, td * 1e3
+
+
+def cpu_baseline(w, moe, budget_s=25.0):
+    """The CPU oracle (port of the reference's naive torch path) on this box's host cores, on a token-subsampled
+    batch of the same layer shape (same H / I / E / k and the same weights)."""
+    import torch
+
+    from oracle import moe_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    c = lambda t: t.detach().to("cpu")
+    ow = O.LayerWeights(
+        c(moe.gate.weight), c(moe._stacks[0]) if moe._stacks else None, None, None,
+        router_b=c(moe.gate.bias) if moe.gate.bias is not None else None,
+    )
+    ow.up_w, ow.down_w = c(moe._stacks[1]), c(moe._stacks[2])
+    if moe.shared_expert is not None:
+        s = moe.shared_expert
+        ow.shared = (c(s.gate_proj.weight), c(s.up_proj.weight), c(s.down_proj.weight))
+
+    def run(tokens):
+        x = torch.randn(tokens, w["H"], generator=torch.Generator().manual_seed(0)).bfloat16()
+        if w["bwd"]:
+            for t in ow.tensors():
+                t.requires_grad_(True)
+                t.grad = None
+            x.requires_grad_(True)
+        t0 = time.perf_counter()
+        out, info = O.moe_forward(x, ow, w["k"], fp8_dispatch=w["fp8"], capacity_factor=w["cap"], capacity_dropless=False,
+                                  aux_coef=0.01 if w["bwd"] else 0.0, training=w["bwd"])
+        if w["bwd"]:
+            loss = (out.float() * torch.ones_like(out, dtype=torch.float32)).sum() + info["aux"]
+            loss.backward()
+        return time.perf_counter() - t0
+
+    tokens = max(w["T"] // 64, 64)
+    t = run(tokens)
+    log(f"[cpu_baseline] {tokens} tokens: {t:.2f} s")
+    if t < budget_s / 8 and tokens * 4 <= w["T"]:
+        tokens *= 4
+        t = run(tokens)
+        log(f"[cpu_baseline] {tokens} tokens: {t:.2f} s")
+    return {
+        "value": tokens / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "sample": f"{tokens} of {w['T']} tokens (same H/I/E/top-k and weights), one {'fwd+bwd' if w['bwd'] else 'fwd'} "
+                  f"pass of the CPU oracle in {t:.2f} s; per-token cost is not linear at this size (the weight reads dominate)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-times", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU (the EP=1 MoE hot path); run with --gpus 1")
+
+    import torch
+
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel.expert_parallel import collect_aux_loss
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device = torch.device("cuda:0")
+    w = WORKLOADS[args.workload]
+    dtype = torch.bfloat16
+    moe = build_layer(w, device, dtype)
+    gx = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn(1, w["T"], w["H"], generator=gx, device=device, dtype=torch.float32).to(dtype)
+    upstream = torch.randn(1, w["T"], w["H"], generator=gx, device=device, dtype=torch.float32).to(dtype)
+    if w["bwd"]:
+        x.requires_grad_(True)
+
+    def step():
+        if w["bwd"]:
+            moe.zero_grad(set_to_none=True)
+            x.grad = None
+            out = moe(x)
+            loss = (out.float() * upstream.float()).sum()
+            aux = collect_aux_loss(moe)
+            if aux is not None:
+                loss = loss + aux
+            loss.backward()
+        else:
+            with torch.no_grad():
+                moe(x)
+
+    timer = GemmTimer()
+    if not args.no_kernel_times:
+        timer.install()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.enabled = not args.no_kernel_times
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    timer.enabled = False
+    tokens_per_s = w["T"] / (ms_per_step * 1e-3)
+    log(f"[bench] {args.workload}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tokens/s")
+
+    result = {
+        "metric": "MoE layer tokens/s fwd+bwd (1 GPU); grouped-GEMM TFLOPS; FP8 quant GB/s",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "tokens": w["T"], "hidden": w["H"], "ffn": w["I"], "experts": w["E"],
+                   "top_k": w["k"], "fp8_dispatch": w["fp8"], "backward": w["bwd"]},
+    }
+
+    if not args.no_kernel_times:
+        # routed rows that reach the expert GEMMs (kept rows under a capacity limit); the shared expert's
+        # launches are timed too but counted with their own row count
+        kt = timer.summary(w["T"] * w["k"], w["H"], w["I"])
+        if w["shared"] or w["cap"] > 0:
+            log("[bench] note: per-launch FLOP assume all routed rows; shared-expert / capacity workloads report time only")
+        kt = {k: (t, f) for k, (t, f, _) in kt.items()}
+        total_ms = sum(t for t, _ in kt.values())
+        total_flop = sum(f for _, f in kt.values())
+        achieved = total_flop / total_ms / 1e9  # TFLOP/s
+        result["roofline"] = {
+            "bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "kernel": "ffn_mfma_kernel (grouped SwiGLU GEMMs: %s)" % ", ".join(kt),
+            "flop_per_step": total_flop, "gemm_ms_per_step": total_ms,
+            "launches": {k: {"ms": t, "tflops": f / t / 1e9} for k, (t, f) in kt.items()},
+        }
+        log(f"[bench] grouped GEMM: {achieved:.0f} TFLOP/s over {total_ms:.2f} ms/step "
+            + " ".join(f"{k}={t:.2f}ms" for k, (t, _) in kt.items()))
+        qg, dg, tq, td = fp8_quant_bandwidth(device)
+        result["fp8_quant"] = {"GBps": qg, "frac_hbm": qg / HBM_PEAK_GBPS, "us": tq, "dequant_GBps": dg,
+                               "dequant_frac_hbm": dg / HBM_PEAK_GBPS, "dequant_us": td,
+                               "shape": "16384 x 4096 bf16 -> e4m3 + fp32 scale, 201392128 B per pass"}
+        log(f"[bench] fp8 quant {qg:.0f} GB/s ({tq:.1f} us), dequant {dg:.0f} GB/s ({td:.1f} us)")
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, moe)
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
