@@ -20,6 +20,8 @@
 // Tiles are enumerated on the device from counts[] (no host copy): expert by expert, N-tile by
 // N-tile, M-tile fastest, and consecutive tiles are handed to the same XCD (block b runs on XCD
 // b % 8) so that the blocks sharing an L2 share operand tiles.
+#include <type_traits>
+
 #include "ffn.h"
 
 namespace {
@@ -58,7 +60,11 @@ struct MfmaParams {
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
 };
 
+#ifdef EXP_NOSWZ
+__device__ __forceinline__ int swz(int) { return 0; }
+#else
 __device__ __forceinline__ int swz(int row) { return (row + (row >> 3)) & 7; }
+#endif
 // X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
 __device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
 
@@ -140,60 +146,67 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         if (!locate_m_grouped(p.counts, p.E, p.n_tiles, &tc)) return;
     }
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS bases and row ranges stay scalar
     const int wm = wave >> 1, wn = wave & 1;
     const int l31 = lane & 31, hi = lane >> 5;
     const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
 
     // ------------------------------------------------------------------------------------------
-    // global -> LDS: per lane, the source of each of the wave's 8 load instructions per operand
+    // global -> LDS: a wave-uniform base pointer per operand plus, per lane, a 32-bit byte offset for each
+    // of the wave's 8 load instructions (scalar base + vector offset addressing: no 64-bit vector adds)
     // ------------------------------------------------------------------------------------------
-    const char* a_src[8];
-    const char* b_src[8];
+    uint32_t a_off[8], b_off[8];
+    const char* a_base;
+    const char* b_base;
     int64_t a_step, b_step;      // bytes per k-tile
     int64_t b_switch_delta = 0;  // dgrad_x: jump from gate_w to up_w half way through K
     int b_switch_kt = 0x7FFFFFFF;
     if (T::kAKMajor) {
         // wave w fills tile rows [64w, 64w+64), 8 rows (128 B each) per instruction
         a_step = BK * 2;
+        a_base = (const char*)(p.A + tc.row0 * p.lda);
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const int r = wave * 64 + q * 8 + (lane >> 3);
             const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the segment re-read its last row (never stored)
-            a_src[q] = (const char*)(p.A + (tc.row0 + ar) * p.lda) + ((lane & 7) ^ swz(r)) * 16;
+            a_off[q] = (uint32_t)(ar * (int)p.lda * 2 + ((lane & 7) ^ swz(r)) * 16);
         }
     } else {
         // wgrad lhs [k rows, P]: wave w fills k rows [16w, 16w+16), 2 rows (512 B each) per instruction
         a_step = BK * p.lda * 2;
+        a_base = (const char*)(p.A + tc.row0 * p.lda);
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             const int kr = wave * 16 + q * 2 + (lane >> 5);
             const int chunk = (lane & 31) ^ swz_x(kr);
             int64_t col = (int64_t)tc.m_tile * BM + chunk * 8;
             col = col + 8 <= p.M ? col : p.M - 8;
-            a_src[q] = (const char*)(p.A + (tc.row0 + kr) * p.lda + col);
+            a_off[q] = (uint32_t)(kr * (int)p.lda * 2 + (int)col * 2);
         }
     }
     if (T::kBKMajor) {
         b_step = BK * 2;
+        int64_t brow0;
+        const uint16_t* bmat;
+        if (MODE == kGateUp) {
+            // B tile rows: per wave column, 64 gate rows then 64 up rows of the same I range -> even waves load
+            // gate rows, odd waves up rows
+            bmat = (wave & 1) ? p.B1 : p.B0;
+            brow0 = (int64_t)tc.n_tile * 128 + (wave >> 1) * 64;
+        } else {
+            bmat = p.B0;
+            brow0 = (int64_t)tc.n_tile * BN + wave * 64;
+        }
+        b_base = (const char*)(bmat + (int64_t)tc.e * p.b_expert_stride + brow0 * p.ldb);
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            const int r = wave * 64 + q * 8 + (lane >> 3);
-            int64_t brow;
-            const uint16_t* bmat;
-            if (MODE == kGateUp) {
-                // B tile rows: per wave column, 64 gate rows then 64 up rows of the same I range
-                bmat = ((r & 127) < 64) ? p.B0 : p.B1;
-                brow = (int64_t)tc.n_tile * 128 + (r >> 7) * 64 + (r & 63);
-            } else {
-                bmat = p.B0;
-                brow = (int64_t)tc.n_tile * BN + r;
-            }
-            b_src[q] = (const char*)(bmat + (int64_t)tc.e * p.b_expert_stride + brow * p.ldb) + ((lane & 7) ^ swz(r)) * 16;
+            const int r = wave * 64 + q * 8 + (lane >> 3);  // row of the LDS tile (fixes the swizzle)
+            b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.ldb * 2 + ((lane & 7) ^ swz(r)) * 16);
         }
     } else {
         b_step = BK * p.ldb * 2;
-        const uint16_t* bmat = MODE == kWgrad ? p.B0 + tc.row0 * p.ldb : p.B0 + (int64_t)tc.e * p.b_expert_stride;
+        b_base = (const char*)(MODE == kWgrad ? p.B0 + tc.row0 * p.ldb : p.B0 + (int64_t)tc.e * p.b_expert_stride);
         if (MODE == kDgradX) {
             b_switch_kt = n_kt / 2;
             b_switch_delta = ((const char*)p.B1 - (const char*)p.B0) - (int64_t)b_switch_kt * b_step;
@@ -204,31 +217,33 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
             const int chunk = (lane & 31) ^ swz_x(kr);
             int64_t col = (int64_t)tc.n_tile * BN + chunk * 8;
             col = col + 8 <= p.N ? col : p.N - 8;
-            b_src[q] = (const char*)(bmat + (int64_t)kr * p.ldb + col);
+            b_off[q] = (uint32_t)(kr * (int)p.ldb * 2 + (int)col * 2);
         }
     }
     // wgrad: k rows past the expert's last row are re-read from its last row and masked out of the fragments
-    auto k_clamp = [&](int kt, int q) -> int64_t {
+    auto k_clamp = [&](int kt, int q) -> int {
         if (MODE != kWgrad) return 0;
         const int kr = kt * BK + wave * 16 + q * 2 + (lane >> 5);
-        return kr < tc.rows ? 0 : (int64_t)(tc.rows - 1 - kr);
+        return kr < tc.rows ? 0 : tc.rows - 1 - kr;
     };
-    auto issue_loads_part = [&](int kt, int stage, int q0) {
+    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq) {
         char* base = lds + stage * kStageBytes;
-        const int64_t b_off = (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
+        const char* ab = a_base + (int64_t)kt * a_step;
+        const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
 #pragma unroll
-        for (int q = q0; q < q0 + 4; ++q) {
-            const int64_t dk = k_clamp(kt, q);
+        for (int q = q0; q < q0 + decltype(nq)::value; ++q) {
+            const int dk = k_clamp(kt, q);
             if (T::kAKMajor)
-                load16_to_lds(a_src[q] + (int64_t)kt * a_step, base + (wave * 64 + q * 8) * 128);
+                load16_to_lds(ab + a_off[q], base + (wave * 64 + q * 8) * 128);
             else
-                load16_to_lds(a_src[q] + (int64_t)kt * a_step + dk * p.lda * 2, base + (wave * 16 + q * 2) * 512);
+                load16_to_lds(ab + (uint32_t)(a_off[q] + dk * (int)p.lda * 2), base + (wave * 16 + q * 2) * 512);
             if (T::kBKMajor)
-                load16_to_lds(b_src[q] + b_off, base + kTileBytes + (wave * 64 + q * 8) * 128);
+                load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * 64 + q * 8) * 128);
             else
-                load16_to_lds(b_src[q] + b_off + dk * p.ldb * 2, base + kTileBytes + (wave * 16 + q * 2) * 512);
+                load16_to_lds(bb + (uint32_t)(b_off[q] + dk * (int)p.ldb * 2), base + kTileBytes + (wave * 16 + q * 2) * 512);
         }
     };
+    auto issue_loads_part = [&](int kt, int stage, int q0) { issue_loads_n(kt, stage, q0, std::integral_constant<int, 4>{}); };
 
     // ------------------------------------------------------------------------------------------
     // LDS -> fragments
@@ -237,29 +252,42 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // X-major: two transpose reads per fragment; lane addresses 8 bytes of k row 16kk + 8*(l>>5) + 4t + ((l>>2)&3)
     //          at column 16*((l>>4)&1) + 4*(l&3) of the 32-column block and receives k rows 16kk + 8*(l>>5) + 4t..+3
     //          of column 16*((l>>4)&1) + (l&15).
-    int a_rd[4], b_rd[4], a_f[4], b_f[4];
+    // Every fragment address is kept in a register (K-major: one per k sub-step and row block, because the
+    // swizzle XORs the chunk index; X-major: one per column block, the k sub-step is an immediate offset) and
+    // flipped between the two stages with one XOR per k-tile: no address arithmetic between the MFMAs.
+    constexpr int kASets = T::kAKMajor ? 4 : 1, kBSets = T::kBKMajor ? 4 : 1;
+    uint32_t a_ad[kASets][4], b_ad[kBSets][4];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
         if (T::kAKMajor) {
             const int ra = wm * 128 + i * 32 + l31;
-            a_rd[i] = ra * 128;
-            a_f[i] = swz(ra);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) a_ad[kk % kASets][i] = lds0 + ra * 128 + (((kk * 2 + hi) ^ swz(ra)) << 4);
         } else {
             const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            a_rd[i] = (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
-            a_f[i] = 0;
+            a_ad[0][i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
         if (T::kBKMajor) {
             const int rb = wn * 128 + i * 32 + l31;
-            b_rd[i] = kTileBytes + rb * 128;
-            b_f[i] = swz(rb);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+                b_ad[kk % kBSets][i] = lds0 + kTileBytes + rb * 128 + (((kk * 2 + hi) ^ swz(rb)) << 4);
         } else {
             const int col = wn * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            b_rd[i] = kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
-            b_f[i] = 0;
+            b_ad[0][i] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
     }
+    auto flip_stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int k2 = 0; k2 < kASets; ++k2) a_ad[k2][i] ^= (uint32_t)kStageBytes;
+#pragma unroll
+            for (int k2 = 0; k2 < kBSets; ++k2) b_ad[k2][i] ^= (uint32_t)kStageBytes;
+        }
+    };
 
     f32x16_t acc[4][4];
 #pragma unroll
@@ -270,24 +298,24 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     bf16x8_t af[2][4], bfr[2][4];
-    auto read_tr_frag = [&](const char* base, int kk) -> bf16x8_t {
-        const s16x4_t lo = lds_read_tr(base + kk * (16 * 512));
-        const s16x4_t hi4 = lds_read_tr(base + kk * (16 * 512) + 4 * 512);
+    auto read_tr_frag = [&](uint32_t ad, int kk) -> bf16x8_t {
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512)));
+        const s16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512) + 4 * 512));
         const s16x8_t v = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
         return __builtin_bit_cast(bf16x8_t, v);
     };
-    auto read_frags = [&](int stage, int kk, int buf) {
-        const char* sb = lds + stage * kStageBytes;
+    // reads the fragments of k sub-step kk from the stage the address registers currently point at
+    auto read_frags = [&](int kk, int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (T::kAKMajor)
-                af[buf][i] = *(const bf16x8_t*)(sb + a_rd[i] + (((kk * 2 + hi) ^ a_f[i]) << 4));
+                af[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)a_ad[kk % kASets][i];
             else
-                af[buf][i] = read_tr_frag(sb + a_rd[i], kk);
+                af[buf][i] = read_tr_frag(a_ad[0][i], kk);
             if (T::kBKMajor)
-                bfr[buf][i] = *(const bf16x8_t*)(sb + b_rd[i] + (((kk * 2 + hi) ^ b_f[i]) << 4));
+                bfr[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)b_ad[kk % kBSets][i];
             else
-                bfr[buf][i] = read_tr_frag(sb + b_rd[i], kk);
+                bfr[buf][i] = read_tr_frag(b_ad[0][i], kk);
         }
     };
     // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
@@ -339,35 +367,58 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        read_frags(0, 0, 0);
+        read_frags(0, 0);
     }
     for (int kt = 0; kt < n_kt; ++kt) {
         const int stage = kt & 1;
         const bool tail = MODE == kWgrad && kt == n_kt - 1;
         __builtin_amdgcn_sched_barrier(0);
+#ifdef EXP_SPREAD4
+        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 0, std::integral_constant<int, 2>{});
+#else
         if (kt > 0 && kt + 1 < n_kt) issue_loads_part(kt + 1, stage ^ 1, 4);  // second half of the refill begun last step
+#endif
         if (tail) mask_tail(kt, 0, 0);
-        read_frags(stage, 1, 1);
+        read_frags(1, 1);
         mma(0);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 1, 1);
-        read_frags(stage, 2, 0);
+#ifdef EXP_SPREAD4
+        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 2, std::integral_constant<int, 2>{});
+#endif
+        read_frags(2, 0);
         mma(1);
+#ifdef EXP_SPREAD4
+        PICOMOE_INTERLEAVE(true)
+#else
         PICOMOE_INTERLEAVE(false)
+#endif
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 2, 0);
-        read_frags(stage, 3, 1);
+#ifdef EXP_SPREAD4
+        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 4, std::integral_constant<int, 2>{});
+#endif
+        read_frags(3, 1);
         mma(0);
+#ifdef EXP_SPREAD4
+        PICOMOE_INTERLEAVE(true)
+#else
         PICOMOE_INTERLEAVE(false)
+#endif
         __builtin_amdgcn_sched_barrier(0);
         // Every wave holds its last fragments of this stage in registers and the next tile has landed:
         // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
+#ifdef EXP_SPREAD4
+        if (kt + 2 < n_kt) issue_loads_n(kt + 2, stage, 6, std::integral_constant<int, 2>{});
+#else
         if (kt + 2 < n_kt) issue_loads_part(kt + 2, stage, 0);
+#endif
         if (tail) mask_tail(kt, 3, 1);
-        if (kt + 1 < n_kt) read_frags(stage ^ 1, 0, 0);
+        flip_stage();
+        if (kt + 1 < n_kt) read_frags(0, 0);
         mma(1);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
