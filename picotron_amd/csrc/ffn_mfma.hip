@@ -60,11 +60,7 @@ struct MfmaParams {
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
 };
 
-#ifdef EXP_NOSWZ
-__device__ __forceinline__ int swz(int) { return 0; }
-#else
 __device__ __forceinline__ int swz(int row) { return (row + (row >> 3)) & 7; }
-#endif
 // X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
 __device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
 
@@ -348,13 +344,18 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
 
     // One k-sub-step = the fragment reads of the NEXT sub-step (and, in two of the four sub-steps, half of the
     // direct-to-LDS loads of a later tile) interleaved with the 16 MFMAs of this sub-step.
+    // Scheduling of one k-sub-step: the LDS reads of the NEXT sub-step (and any direct-to-LDS loads) go into
+    // the first half, one after each MFMA (the sub-step starts with an MFMA: the compiler waits for ALL LDS
+    // reads before a sub-step's first MFMA, so no read may sit right in front of it), and the second half
+    // (8 MFMAs, 256 cycles) covers their latency.
     constexpr int kReadsPerGroup = ((T::kAKMajor ? 4 : 8) + (T::kBKMajor ? 4 : 8)) / 8;
 #define PICOMOE_INTERLEAVE(WITH_LOADS)                                            \
     _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                            \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        \
         __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerGroup, 0);           \
         if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                        \
-    }
+    }                                                                             \
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
 
     if (n_kt > 0) {
         issue_loads_part(0, 0, 0);
@@ -373,57 +374,41 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         const int stage = kt & 1;
         const bool tail = MODE == kWgrad && kt == n_kt - 1;
         __builtin_amdgcn_sched_barrier(0);
-#ifdef EXP_SPREAD4
-        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 0, std::integral_constant<int, 2>{});
-#else
-        if (kt > 0 && kt + 1 < n_kt) issue_loads_part(kt + 1, stage ^ 1, 4);  // second half of the refill begun last step
-#endif
+        // second half of the refill begun in the previous k-step.  Issued unconditionally (past the end the tile
+        // index is clamped and the data land in a stage nobody reads) so that the loads sit in the same basic
+        // block as the MFMAs and can be interleaved with them.
+        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 4);
         if (tail) mask_tail(kt, 0, 0);
         read_frags(1, 1);
         mma(0);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 1, 1);
-#ifdef EXP_SPREAD4
-        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 2, std::integral_constant<int, 2>{});
-#endif
         read_frags(2, 0);
         mma(1);
-#ifdef EXP_SPREAD4
-        PICOMOE_INTERLEAVE(true)
-#else
         PICOMOE_INTERLEAVE(false)
-#endif
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 2, 0);
-#ifdef EXP_SPREAD4
-        if (kt + 1 < n_kt) issue_loads_n(kt + 1, stage ^ 1, 4, std::integral_constant<int, 2>{});
-#endif
         read_frags(3, 1);
         mma(0);
-#ifdef EXP_SPREAD4
-        PICOMOE_INTERLEAVE(true)
-#else
         PICOMOE_INTERLEAVE(false)
-#endif
         __builtin_amdgcn_sched_barrier(0);
         // Every wave holds its last fragments of this stage in registers and the next tile has landed:
         // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-#ifdef EXP_SPREAD4
-        if (kt + 2 < n_kt) issue_loads_n(kt + 2, stage, 6, std::integral_constant<int, 2>{});
-#else
-        if (kt + 2 < n_kt) issue_loads_part(kt + 2, stage, 0);
-#endif
+        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0);
         if (tail) mask_tail(kt, 3, 1);
         flip_stage();
-        if (kt + 1 < n_kt) read_frags(0, 0);
+        read_frags(0, 0);  // past the last tile this reads a stage that is not used any more
         mma(1);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
     }
 #undef PICOMOE_INTERLEAVE
+    // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
 
     // ------------------------------------------------------------------------------------------
     // epilogue.  A lane holds column (l & 31) and rows 8*(r/4) + 4*(l >> 5) + (r % 4) of each 32 x 32
