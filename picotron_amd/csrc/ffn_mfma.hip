@@ -30,6 +30,10 @@ constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kTileBytes = 256 * BK * 2;  // 32 KB per operand tile
 constexpr int kStageBytes = 2 * kTileBytes;
 constexpr int kNumXcd = 8;
+#ifndef PICOMOE_MFMA_WAVES
+#define PICOMOE_MFMA_WAVES 8
+#endif
+constexpr int kWaves = PICOMOE_MFMA_WAVES;
 
 enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
 
@@ -131,9 +135,18 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
     return true;
 }
 
-template <int MODE>
-__global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
+// NW wavefronts per block: 4 (one per SIMD, wave tile 128 x 128) or 8 (two per SIMD, wave tile 128 x 64, so that
+// one wave's waits and memory instructions are covered by the other wave's MFMAs).
+template <int MODE, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
+    constexpr int NI = 4;               // 32-row blocks per wave
+    constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
+    constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
+    constexpr int CW = NJ * 32;         // columns per wave
+    constexpr int QN = 32 / NW;         // direct-to-LDS load instructions per operand, wave and k-tile
+    constexpr int RPW = QN * 8;         // K-major tile rows a wave fills
+    constexpr int KPW = QN * 2;         // X-major k rows a wave fills
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
     if (MODE == kWgrad) {
@@ -144,7 +157,7 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS bases and row ranges stay scalar
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / kWaveCols, wn = wave % kWaveCols;
     const int l31 = lane & 31, hi = lane >> 5;
     const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
 
@@ -152,29 +165,29 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // global -> LDS: a wave-uniform base pointer per operand plus, per lane, a 32-bit byte offset for each
     // of the wave's 8 load instructions (scalar base + vector offset addressing: no 64-bit vector adds)
     // ------------------------------------------------------------------------------------------
-    uint32_t a_off[8], b_off[8];
+    uint32_t a_off[QN], b_off[QN];
     const char* a_base;
     const char* b_base;
     int64_t a_step, b_step;      // bytes per k-tile
     int64_t b_switch_delta = 0;  // dgrad_x: jump from gate_w to up_w half way through K
     int b_switch_kt = 0x7FFFFFFF;
     if (T::kAKMajor) {
-        // wave w fills tile rows [64w, 64w+64), 8 rows (128 B each) per instruction
+        // wave w fills tile rows [RPW*w, RPW*(w+1)), 8 rows (128 B each) per instruction
         a_step = BK * 2;
         a_base = (const char*)(p.A + tc.row0 * p.lda);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const int r = wave * 64 + q * 8 + (lane >> 3);
+        for (int q = 0; q < QN; ++q) {
+            const int r = wave * RPW + q * 8 + (lane >> 3);
             const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the segment re-read its last row (never stored)
             a_off[q] = (uint32_t)(ar * (int)p.lda * 2 + ((lane & 7) ^ swz(r)) * 16);
         }
     } else {
-        // wgrad lhs [k rows, P]: wave w fills k rows [16w, 16w+16), 2 rows (512 B each) per instruction
+        // wgrad lhs [k rows, P]: wave w fills k rows [KPW*w, KPW*(w+1)), 2 rows (512 B each) per instruction
         a_step = BK * p.lda * 2;
         a_base = (const char*)(p.A + tc.row0 * p.lda);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const int kr = wave * 16 + q * 2 + (lane >> 5);
+        for (int q = 0; q < QN; ++q) {
+            const int kr = wave * KPW + q * 2 + (lane >> 5);
             const int chunk = (lane & 31) ^ swz_x(kr);
             int64_t col = (int64_t)tc.m_tile * BM + chunk * 8;
             col = col + 8 <= p.M ? col : p.M - 8;
@@ -186,18 +199,19 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         int64_t brow0;
         const uint16_t* bmat;
         if (MODE == kGateUp) {
-            // B tile rows: per wave column, 64 gate rows then 64 up rows of the same I range -> even waves load
-            // gate rows, odd waves up rows
+            // B tile rows: per wave column (CW rows), CW/2 gate rows then CW/2 up rows of the same I range.
+            // RPW == CW/2, so even waves load gate rows and odd waves up rows.
+            static_assert(RPW * 2 == CW, "gate/up interleave assumes one wave loads half a wave column");
             bmat = (wave & 1) ? p.B1 : p.B0;
-            brow0 = (int64_t)tc.n_tile * 128 + (wave >> 1) * 64;
+            brow0 = (int64_t)tc.n_tile * 128 + (wave >> 1) * (CW / 2);
         } else {
             bmat = p.B0;
-            brow0 = (int64_t)tc.n_tile * BN + wave * 64;
+            brow0 = (int64_t)tc.n_tile * BN + wave * RPW;
         }
         b_base = (const char*)(bmat + (int64_t)tc.e * p.b_expert_stride + brow0 * p.ldb);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const int r = wave * 64 + q * 8 + (lane >> 3);  // row of the LDS tile (fixes the swizzle)
+        for (int q = 0; q < QN; ++q) {
+            const int r = wave * RPW + q * 8 + (lane >> 3);  // row of the LDS tile (fixes the swizzle)
             b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.ldb * 2 + ((lane & 7) ^ swz(r)) * 16);
         }
     } else {
@@ -208,8 +222,8 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
             b_switch_delta = ((const char*)p.B1 - (const char*)p.B0) - (int64_t)b_switch_kt * b_step;
         }
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const int kr = wave * 16 + q * 2 + (lane >> 5);
+        for (int q = 0; q < QN; ++q) {
+            const int kr = wave * KPW + q * 2 + (lane >> 5);
             const int chunk = (lane & 31) ^ swz_x(kr);
             int64_t col = (int64_t)tc.n_tile * BN + chunk * 8;
             col = col + 8 <= p.N ? col : p.N - 8;
@@ -219,7 +233,7 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // wgrad: k rows past the expert's last row are re-read from its last row and masked out of the fragments
     auto k_clamp = [&](int kt, int q) -> int {
         if (MODE != kWgrad) return 0;
-        const int kr = kt * BK + wave * 16 + q * 2 + (lane >> 5);
+        const int kr = kt * BK + wave * KPW + q * 2 + (lane >> 5);
         return kr < tc.rows ? 0 : tc.rows - 1 - kr;
     };
     auto issue_loads_n = [&](int kt, int stage, int q0, auto nq) {
@@ -230,16 +244,19 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         for (int q = q0; q < q0 + decltype(nq)::value; ++q) {
             const int dk = k_clamp(kt, q);
             if (T::kAKMajor)
-                load16_to_lds(ab + a_off[q], base + (wave * 64 + q * 8) * 128);
+                load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
             else
-                load16_to_lds(ab + (uint32_t)(a_off[q] + dk * (int)p.lda * 2), base + (wave * 16 + q * 2) * 512);
+                load16_to_lds(ab + (uint32_t)(a_off[q] + dk * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
             if (T::kBKMajor)
-                load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * 64 + q * 8) * 128);
+                load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * RPW + q * 8) * 128);
             else
-                load16_to_lds(bb + (uint32_t)(b_off[q] + dk * (int)p.ldb * 2), base + kTileBytes + (wave * 16 + q * 2) * 512);
+                load16_to_lds(bb + (uint32_t)(b_off[q] + dk * (int)p.ldb * 2), base + kTileBytes + (wave * KPW + q * 2) * 512);
         }
     };
-    auto issue_loads_part = [&](int kt, int stage, int q0) { issue_loads_n(kt, stage, q0, std::integral_constant<int, 4>{}); };
+    // half of a wave's loads for one tile: part 0 or 1
+    auto issue_loads_part = [&](int kt, int stage, int part) {
+        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{});
+    };
 
     // ------------------------------------------------------------------------------------------
     // LDS -> fragments
@@ -252,11 +269,11 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // swizzle XORs the chunk index; X-major: one per column block, the k sub-step is an immediate offset) and
     // flipped between the two stages with one XOR per k-tile: no address arithmetic between the MFMAs.
     constexpr int kASets = T::kAKMajor ? 4 : 1, kBSets = T::kBKMajor ? 4 : 1;
-    uint32_t a_ad[kASets][4], b_ad[kBSets][4];
+    uint32_t a_ad[kASets][NI], b_ad[kBSets][NJ];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+    const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
+    for (int i = 0; i < NI; ++i) {
         if (T::kAKMajor) {
             const int ra = wm * 128 + i * 32 + l31;
 #pragma unroll
@@ -265,35 +282,39 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
             const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
             a_ad[0][i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
         if (T::kBKMajor) {
-            const int rb = wn * 128 + i * 32 + l31;
+            const int rb = wn * CW + j * 32 + l31;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk)
-                b_ad[kk % kBSets][i] = lds0 + kTileBytes + rb * 128 + (((kk * 2 + hi) ^ swz(rb)) << 4);
+                b_ad[kk % kBSets][j] = lds0 + kTileBytes + rb * 128 + (((kk * 2 + hi) ^ swz(rb)) << 4);
         } else {
-            const int col = wn * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            b_ad[0][i] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            const int col = wn * CW + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            b_ad[0][j] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
     }
     auto flip_stage = [&]() {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int k2 = 0; k2 < kASets; ++k2)
 #pragma unroll
-            for (int k2 = 0; k2 < kASets; ++k2) a_ad[k2][i] ^= (uint32_t)kStageBytes;
+            for (int i = 0; i < NI; ++i) a_ad[k2][i] ^= (uint32_t)kStageBytes;
 #pragma unroll
-            for (int k2 = 0; k2 < kBSets; ++k2) b_ad[k2][i] ^= (uint32_t)kStageBytes;
-        }
+        for (int k2 = 0; k2 < kBSets; ++k2)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) b_ad[k2][j] ^= (uint32_t)kStageBytes;
     };
 
-    f32x16_t acc[4][4];
+    f32x16_t acc[NI][NJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    bf16x8_t af[2][4], bfr[2][4];
+    bf16x8_t af[2][NI], bfr[2][NJ];
     auto read_tr_frag = [&](uint32_t ad, int kk) -> bf16x8_t {
         const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512)));
         const s16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512) + 4 * 512));
@@ -303,15 +324,18 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // reads the fragments of k sub-step kk from the stage the address registers currently point at
     auto read_frags = [&](int kk, int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NI; ++i) {
             if (T::kAKMajor)
                 af[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)a_ad[kk % kASets][i];
             else
                 af[buf][i] = read_tr_frag(a_ad[0][i], kk);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
             if (T::kBKMajor)
-                bfr[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)b_ad[kk % kBSets][i];
+                bfr[buf][j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)b_ad[kk % kBSets][j];
             else
-                bfr[buf][i] = read_tr_frag(b_ad[0][i], kk);
+                bfr[buf][j] = read_tr_frag(b_ad[0][j], kk);
         }
     };
     // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
@@ -319,26 +343,23 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         if (MODE != kWgrad) return;
         const int valid = tc.rows - kt * BK - kk * 16 - 8 * hi;  // lane holds k = 8*hi + 0..7 of this sub-step
         if (valid >= 8) return;
+        auto zero_tail = [&](bf16x8_t& f) {
+            s16x8_t a = __builtin_bit_cast(s16x8_t, f);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            s16x8_t a = __builtin_bit_cast(s16x8_t, af[buf][i]);
-            s16x8_t b = __builtin_bit_cast(s16x8_t, bfr[buf][i]);
+            for (int e = 0; e < 8; ++e)
+                if (e >= valid) a[e] = 0;
+            f = __builtin_bit_cast(bf16x8_t, a);
+        };
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (e >= valid) {
-                    a[e] = 0;
-                    b[e] = 0;
-                }
-            }
-            af[buf][i] = __builtin_bit_cast(bf16x8_t, a);
-            bfr[buf][i] = __builtin_bit_cast(bf16x8_t, b);
-        }
+        for (int i = 0; i < NI; ++i) zero_tail(af[buf][i]);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) zero_tail(bfr[buf][j]);
     };
     auto mma = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < NJ; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
     };
 
@@ -348,22 +369,27 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
     // the first half, one after each MFMA (the sub-step starts with an MFMA: the compiler waits for ALL LDS
     // reads before a sub-step's first MFMA, so no read may sit right in front of it), and the second half
     // (8 MFMAs, 256 cycles) covers their latency.
-    constexpr int kReadsPerGroup = ((T::kAKMajor ? 4 : 8) + (T::kBKMajor ? 4 : 8)) / 8;
+    constexpr int kReads = NI * (T::kAKMajor ? 1 : 2) + NJ * (T::kBKMajor ? 1 : 2);  // LDS reads per sub-step
+    constexpr int kMfmas = NI * NJ;
+    constexpr int kGroups = kMfmas / 2;                                               // MFMAs that get company
+    constexpr int kReadsPerGroup = (kReads + kGroups - 1) / kGroups;
 #define PICOMOE_INTERLEAVE(WITH_LOADS)                                            \
-    _Pragma("unroll") for (int s_ = 0; s_ < 8; ++s_) {                            \
+    _Pragma("unroll") for (int s_ = 0; s_ < kGroups; ++s_) {                      \
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        \
         __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerGroup, 0);           \
         if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
     }                                                                             \
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kGroups, 0);
 
     if (n_kt > 0) {
         issue_loads_part(0, 0, 0);
-        issue_loads_part(0, 0, 4);
+        issue_loads_part(0, 0, 1);
         if (n_kt > 1) {
             issue_loads_part(1, 1, 0);
-            issue_loads_part(1, 1, 4);
-            __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 landed, tile 1 may still be in flight
+            issue_loads_part(1, 1, 1);
+            // vmcnt(2*QN): tile 0 landed, tile 1 may still be in flight
+            if (QN == 8) __builtin_amdgcn_s_waitcnt(0x4F70);
+            else __builtin_amdgcn_s_waitcnt(0x0F78);
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
@@ -377,7 +403,7 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         // second half of the refill begun in the previous k-step.  Issued unconditionally (past the end the tile
         // index is clamped and the data land in a stage nobody reads) so that the loads sit in the same basic
         // block as the MFMAs and can be interleaved with them.
-        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 4);
+        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1);
         if (tail) mask_tail(kt, 0, 0);
         read_frags(1, 1);
         mma(0);
@@ -424,11 +450,12 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
         valid_rows = left < BM ? (int)left : BM;
         out_row0 = (int64_t)tc.e * p.M + (int64_t)tc.m_tile * BM;
     }
-    constexpr int kEpiCols = MODE == kGateUp ? 64 : 128;  // output columns per wave and pass
+    constexpr int kEpiCols = MODE == kGateUp ? CW / 2 : CW;  // output columns per wave and pass
     constexpr int kEpiStride = (kEpiCols + 8) * 2;        // bytes; the 16-byte pad rotates rows over the banks
     char* epi = lds + wave * (32 * kEpiStride);
     constexpr int kChunksPerRow = kEpiCols / 8;
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
+    static_assert(kReadIters >= 1, "a pass must cover at least one chunk per lane");
 
     auto stage_block = [&](auto value) {  // value(j, r) -> float, j over the 32-column blocks of this pass
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // earlier read-backs of this slice are done
@@ -455,30 +482,30 @@ __global__ __launch_bounds__(256, 1) void ffn_mfma_kernel(MfmaParams p) {
 
     if (MODE == kGateUp) {
         const int64_t I = p.N;
-        const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * 64;
+        const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NI; ++i) {
             // g and u rounded to bf16 in place (what the reference's two Linear outputs hold)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][r]));
             stage_block([&](int j, int r) {
-                const float g = acc[i][j][r], u = acc[i][j + 2][r];
+                const float g = acc[i][j][r], u = acc[i][j + NJ / 2][r];
                 return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
             });
             for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v; });
             if (p.out2) {
                 stage_block([&](int j, int r) { return acc[i][j][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v; });
-                stage_block([&](int j, int r) { return acc[i][j + 2][r]; });
+                stage_block([&](int j, int r) { return acc[i][j + NJ / 2][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v; });
             }
         }
     } else {
-        const int64_t col0 = (int64_t)tc.n_tile * BN + wn * 128;
+        const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NI; ++i) {
             stage_block([&](int j, int r) { return acc[i][j][r]; });
             for_chunks(i, [&](int trow, int c, u32x4_t v) {
                 const int64_t col = col0 + c;
@@ -550,7 +577,7 @@ int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const
     p.A = (const uint16_t*)x; p.lda = s.H;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;
     p.out = (uint16_t*)act; p.ldo = s.I; p.out2 = (uint16_t*)inter13;
-    hipLaunchKernelGGL(ffn_mfma_kernel<kGateUp>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kGateUp, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -560,7 +587,7 @@ int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const 
     p.A = (const uint16_t*)act; p.lda = s.I;
     p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;
     p.out = (uint16_t*)y; p.ldo = s.H; p.aux = (const uint16_t*)row_weight;
-    hipLaunchKernelGGL(ffn_mfma_kernel<kDown>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDown, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -571,7 +598,7 @@ int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, co
     p.A = (const uint16_t*)dy; p.lda = s.H;
     p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;  // down_w[e] read as [K = H][N = I]
     p.out = (uint16_t*)d_inter13; p.ldo = 2 * s.I; p.out2 = (uint16_t*)act_out; p.aux = (const uint16_t*)inter13;
-    hipLaunchKernelGGL(ffn_mfma_kernel<kDgradAct>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradAct, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -582,7 +609,7 @@ int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_
     p.A = (const uint16_t*)d_inter13; p.lda = 2 * s.I;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;  // [K = I][N = H]
     p.out = (uint16_t*)dx; p.ldo = s.H;
-    hipLaunchKernelGGL(ffn_mfma_kernel<kDgradX>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradX, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -600,6 +627,6 @@ int ffn_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const voi
     p.B0 = (const uint16_t*)rhs; p.ldb = ld_rhs;
     p.out = (uint16_t*)out; p.ldo = Q;
     const int64_t tiles = (int64_t)s.E * p.m_tiles * p.n_tiles;
-    hipLaunchKernelGGL(ffn_mfma_kernel<kWgrad>, dim3(round_up_xcd(tiles)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kWgrad, kWaves>), dim3(round_up_xcd(tiles)), dim3(kWaves * 64), 0, st, p);
     return picomoe_launch_status();
 }
