@@ -93,18 +93,41 @@ __device__ __forceinline__ int64_t logical_tile(int64_t total) {
     return L < total ? L : -1;
 }
 
+// M-grouped tiles come in two classes.  Heavy: full 256-row tiles and tails of more than 128 rows.  Light: tails
+// of at most 128 rows, which cost about half (the wavefronts owning rows 128..255 skip their MFMAs).  Every XCD
+// gets a contiguous run of the heavy tiles followed by a run of the light ones, so the light tiles fill the last,
+// partly occupied round of blocks instead of a full-cost tile being left over there.
 __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, TileCoord* tc) {
-    int64_t total_m = 0;
-    for (int e = 0; e < E; ++e) total_m += (counts[e] + BM - 1) / BM;
-    int64_t L = logical_tile(total_m * n_tiles);
-    if (L < 0) return false;
+    int64_t heavy_m = 0, light_m = 0;
+    for (int e = 0; e < E; ++e) {
+        const int64_t c = counts[e], rem = c % BM;
+        heavy_m += c / BM + (rem > BM / 2);
+        light_m += (rem > 0 && rem <= BM / 2);
+    }
+    const int64_t heavy = heavy_m * n_tiles, light = light_m * n_tiles;
+    const int64_t heavy_per_xcd = (heavy + kNumXcd - 1) / kNumXcd, light_per_xcd = (light + kNumXcd - 1) / kNumXcd;
+    const int64_t xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    bool want_light;
+    int64_t L;
+    if (slot < heavy_per_xcd) {
+        want_light = false;
+        L = xcd * heavy_per_xcd + slot;
+        if (L >= heavy) return false;
+    } else if (slot - heavy_per_xcd < light_per_xcd) {
+        want_light = true;
+        L = xcd * light_per_xcd + (slot - heavy_per_xcd);
+        if (L >= light) return false;
+    } else {
+        return false;
+    }
     int64_t start = 0;
     for (int e = 0; e < E; ++e) {
-        const int64_t c = counts[e];
-        const int64_t me = (c + BM - 1) / BM;
+        const int64_t c = counts[e], full = c / BM, rem = c % BM;
+        const bool light_tail = rem > 0 && rem <= BM / 2;
+        const int64_t me = want_light ? (int64_t)light_tail : full + (rem > BM / 2);
         const int64_t te = me * n_tiles;
         if (L < te) {
-            const int m = (int)(L % me);
+            const int m = want_light ? (int)full : (int)(L % me);
             tc->e = e;
             tc->m_tile = m;
             tc->n_tile = (int)(L / me);
@@ -160,6 +183,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
     const int l31 = lane & 31, hi = lane >> 5;
     const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
+    // a wavefront whose 128 rows all lie past the end of the expert's segment keeps loading and synchronising
+    // but skips its fragment reads and MFMAs
+    const bool wave_active = MODE == kWgrad || wm * 128 < tc.rows;
 
     // ------------------------------------------------------------------------------------------
     // global -> LDS: a wave-uniform base pointer per operand plus, per lane, a 32-bit byte offset for each
@@ -236,7 +262,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         const int kr = kt * BK + wave * KPW + q * 2 + (lane >> 5);
         return kr < tc.rows ? 0 : tc.rows - 1 - kr;
     };
-    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq) {
+    // `full` (a std::bool_constant): the tile has all 256 rows, so the per-wave / per-row checks vanish at compile time
+    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq, auto /*full*/) {
         char* base = lds + stage * kStageBytes;
         const char* ab = a_base + (int64_t)kt * a_step;
         const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
@@ -254,8 +281,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     };
     // half of a wave's loads for one tile: part 0 or 1
-    auto issue_loads_part = [&](int kt, int stage, int part) {
-        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{});
+    auto issue_loads_part = [&](int kt, int stage, int part, auto full) {
+        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{}, full);
     };
 
     // ------------------------------------------------------------------------------------------
@@ -265,45 +292,38 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // X-major: two transpose reads per fragment; lane addresses 8 bytes of k row 16kk + 8*(l>>5) + 4t + ((l>>2)&3)
     //          at column 16*((l>>4)&1) + 4*(l&3) of the 32-column block and receives k rows 16kk + 8*(l>>5) + 4t..+3
     //          of column 16*((l>>4)&1) + (l&15).
-    // Every fragment address is kept in a register (K-major: one per k sub-step and row block, because the
-    // swizzle XORs the chunk index; X-major: one per column block, the k sub-step is an immediate offset) and
-    // flipped between the two stages with one XOR per k-tile: no address arithmetic between the MFMAs.
-    constexpr int kASets = T::kAKMajor ? 4 : 1, kBSets = T::kBKMajor ? 4 : 1;
-    uint32_t a_ad[kASets][NI], b_ad[kBSets][NJ];
+    // One address register per fragment block, pointing at k sub-step 0 of the current stage.  K-major: the
+    // swizzle XORs the chunk index, and (2kk + hi) ^ f == (hi ^ f) ^ 2kk, so sub-step kk is that address XOR
+    // (kk << 5) -- one VALU op at the use; X-major: the sub-step is an immediate offset.  One XOR per register
+    // and k-tile flips between the two stages.
+    uint32_t a_ad[NI], b_ad[NJ];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
     const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
         if (T::kAKMajor) {
             const int ra = wm * 128 + i * 32 + l31;
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) a_ad[kk % kASets][i] = lds0 + ra * 128 + (((kk * 2 + hi) ^ swz(ra)) << 4);
+            a_ad[i] = lds0 + ra * 128 + ((hi ^ swz(ra)) << 4);
         } else {
             const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            a_ad[0][i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            a_ad[i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
     }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         if (T::kBKMajor) {
             const int rb = wn * CW + j * 32 + l31;
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk)
-                b_ad[kk % kBSets][j] = lds0 + kTileBytes + rb * 128 + (((kk * 2 + hi) ^ swz(rb)) << 4);
+            b_ad[j] = lds0 + kTileBytes + rb * 128 + ((hi ^ swz(rb)) << 4);
         } else {
             const int col = wn * CW + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            b_ad[0][j] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            b_ad[j] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
     }
     auto flip_stage = [&]() {
 #pragma unroll
-        for (int k2 = 0; k2 < kASets; ++k2)
+        for (int i = 0; i < NI; ++i) a_ad[i] ^= (uint32_t)kStageBytes;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) a_ad[k2][i] ^= (uint32_t)kStageBytes;
-#pragma unroll
-        for (int k2 = 0; k2 < kBSets; ++k2)
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) b_ad[k2][j] ^= (uint32_t)kStageBytes;
+        for (int j = 0; j < NJ; ++j) b_ad[j] ^= (uint32_t)kStageBytes;
     };
 
     f32x16_t acc[NI][NJ];
@@ -322,20 +342,21 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         return __builtin_bit_cast(bf16x8_t, v);
     };
     // reads the fragments of k sub-step kk from the stage the address registers currently point at
-    auto read_frags = [&](int kk, int buf) {
+    auto read_frags = [&](int kk, int buf, auto full) {
+        if (!decltype(full)::value && !wave_active) return;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             if (T::kAKMajor)
-                af[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)a_ad[kk % kASets][i];
+                af[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(a_ad[i] ^ (uint32_t)(kk << 5));
             else
-                af[buf][i] = read_tr_frag(a_ad[0][i], kk);
+                af[buf][i] = read_tr_frag(a_ad[i], kk);
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             if (T::kBKMajor)
-                bfr[buf][j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)b_ad[kk % kBSets][j];
+                bfr[buf][j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(b_ad[j] ^ (uint32_t)(kk << 5));
             else
-                bfr[buf][j] = read_tr_frag(b_ad[0][j], kk);
+                bfr[buf][j] = read_tr_frag(b_ad[j], kk);
         }
     };
     // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
@@ -355,7 +376,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) zero_tail(bfr[buf][j]);
     };
-    auto mma = [&](int buf) {
+    auto mma = [&](int buf, auto full) {
+        if (!decltype(full)::value && !wave_active) return;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -382,20 +404,21 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kGroups, 0);
 
     if (n_kt > 0) {
-        issue_loads_part(0, 0, 0);
-        issue_loads_part(0, 0, 1);
+        issue_loads_part(0, 0, 0, std::false_type{});
+        issue_loads_part(0, 0, 1, std::false_type{});
         if (n_kt > 1) {
-            issue_loads_part(1, 1, 0);
-            issue_loads_part(1, 1, 1);
-            // vmcnt(2*QN): tile 0 landed, tile 1 may still be in flight
+            issue_loads_part(1, 1, 0, std::false_type{});
+            issue_loads_part(1, 1, 1, std::false_type{});
+            // vmcnt(2*QN): tile 0 has landed, tile 1 may still be in flight
             if (QN == 8) __builtin_amdgcn_s_waitcnt(0x4F70);
             else __builtin_amdgcn_s_waitcnt(0x0F78);
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        read_frags(0, 0);
+        read_frags(0, 0, std::false_type{});
     }
+    auto k_loop = [&](auto full) {
     for (int kt = 0; kt < n_kt; ++kt) {
         const int stage = kt & 1;
         const bool tail = MODE == kWgrad && kt == n_kt - 1;
@@ -403,34 +426,38 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         // second half of the refill begun in the previous k-step.  Issued unconditionally (past the end the tile
         // index is clamped and the data land in a stage nobody reads) so that the loads sit in the same basic
         // block as the MFMAs and can be interleaved with them.
-        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1);
+        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1, full);
         if (tail) mask_tail(kt, 0, 0);
-        read_frags(1, 1);
-        mma(0);
+        read_frags(1, 1, full);
+        mma(0, full);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 1, 1);
-        read_frags(2, 0);
-        mma(1);
+        read_frags(2, 0, full);
+        mma(1, full);
         PICOMOE_INTERLEAVE(false)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 2, 0);
-        read_frags(3, 1);
-        mma(0);
+        read_frags(3, 1, full);
+        mma(0, full);
         PICOMOE_INTERLEAVE(false)
         __builtin_amdgcn_sched_barrier(0);
         // Every wave holds its last fragments of this stage in registers and the next tile has landed:
         // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0);
+        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0, full);
         if (tail) mask_tail(kt, 3, 1);
         flip_stage();
-        read_frags(0, 0);  // past the last tile this reads a stage that is not used any more
-        mma(1);
+        read_frags(0, 0, full);  // past the last tile this reads a stage that is not used any more
+        mma(1, full);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
     }
+    };
+    // two copies of the loop: full tiles (the common case) run without any per-wave checks
+    if (MODE == kWgrad || tc.rows >= BM) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
 #undef PICOMOE_INTERLEAVE
     // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -552,8 +579,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 }
 
 inline unsigned round_up_xcd(int64_t g) { return (unsigned)(((g + kNumXcd - 1) / kNumXcd) * kNumXcd); }
+// upper bound of 8 * (ceil(heavy / 8) + ceil(light / 8)) over every split of the rows among the experts
 inline unsigned grid_m_grouped(const FfnShape& s, int n_tiles) {
-    return round_up_xcd((s.n_rows / BM + s.E) * (int64_t)n_tiles);
+    return round_up_xcd((s.n_rows / BM + s.E) * (int64_t)n_tiles) + 2 * kNumXcd;
 }
 
 MfmaParams base_params(const FfnShape& s) {
