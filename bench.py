@@ -92,6 +92,7 @@ class GemmTimer:
         self.records = []
         self.enabled = False
         self.pool = []
+        self.shared_mult = 1
 
     def prepare(self, n_events):
         """Create the events before the clock starts (creating one costs far more than recording it)."""
@@ -117,7 +118,12 @@ class GemmTimer:
                 label = name
                 if name == "wgrad":  # (lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset)
                     label = "wgrad_down" if a[1] == a[7] else ("wgrad_up" if kw.get("lhs_offset", 0) else "wgrad_gate")
-                self.records.append((label, name, st, en))
+                    n_experts, rows = a[5], a[6]
+                else:  # (x, counts, weight, ...): weight [E, ., .]
+                    n_experts, rows = a[2].shape[0], a[0].shape[0]
+                if n_experts == 1:
+                    label = "shared_" + label  # the shared expert runs the same kernels with one expert
+                self.records.append((label, name, st, en, rows))
                 return out
             return timed
 
@@ -126,8 +132,11 @@ class GemmTimer:
 
     def summary(self, routed_rows, H, I):
         per = {}
-        for label, name, st, en in self.records:
-            d = per.setdefault(label, {"ms": 0.0, "n": 0, "flop": self.FLOP[name] * routed_rows * H * I})
+        for label, name, st, en, rows in self.records:
+            # routed launches: the rows that reach the GEMMs (kept rows under a capacity limit); shared: all tokens
+            n_rows = rows if label.startswith("shared_") else routed_rows
+            i_dim = I * self.shared_mult if label.startswith("shared_") else I
+            d = per.setdefault(label, {"ms": 0.0, "n": 0, "flop": self.FLOP[name] * n_rows * H * i_dim})
             d["ms"] += st.elapsed_time(en)
             d["n"] += 1
         return {k: (v["ms"] / v["n"], v["flop"], v["n"]) for k, v in per.items()}
@@ -283,9 +292,18 @@ def main():
     if not args.no_kernel_times:
         # routed rows that reach the expert GEMMs (kept rows under a capacity limit); the shared expert's
         # launches are timed too but counted with their own row count
-        kt = timer.summary(w["T"] * w["k"], w["H"], w["I"])
-        if w["shared"] or w["cap"] > 0:
-            log("[bench] note: per-launch FLOP assume all routed rows; shared-expert / capacity workloads report time only")
+        routed_rows = w["T"] * w["k"]
+        if w["cap"] > 0:  # count the kept rows from the drop mask, not the routed ones
+            from picotron_amd import _ops
+            from picotron_amd.expert_parallel.capacity_moe import compute_capacity
+
+            with torch.no_grad():
+                idx, _ = moe._route(x.reshape(-1, w["H"]))
+                plan = _ops.permute_plan(idx.reshape(-1), w["E"], capacity=compute_capacity(w["T"], w["k"], w["E"], w["cap"]))
+                routed_rows = int(plan.kept_counts.sum().item())
+            result["config"]["kept_rows"] = routed_rows
+        timer.shared_mult = max(w["shared"], 1)
+        kt = timer.summary(routed_rows, w["H"], w["I"])
         kt = {k: (t, f) for k, (t, f, _) in kt.items()}
         total_ms = sum(t for t, _ in kt.values())
         total_flop = sum(f for _, f in kt.values())

@@ -64,7 +64,9 @@ struct MfmaParams {
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
 };
 
-__device__ __forceinline__ int swz(int row) { return (row + (row >> 3)) & 7; }
+__device__ __forceinline__ int swz(int row) {
+    return (row + (row >> 3)) & 7;
+}
 // X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
 __device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
 

@@ -275,3 +275,91 @@ def test_capacity_moe_function_signature(gpu):
     within, counts = _slot_assignment(idx.reshape(-1).cuda(), E)
     rw, rc = O.slot_assignment(idx.reshape(-1), E)
     assert torch.equal(within.cpu(), rw) and torch.equal(counts.cpu(), rc)
+
+
+def _sample_check(moe, x_tokens, out, idx, wts, keep, sample, rtol):
+    """Per-token brute force on the CPU for a sample of tokens: each kept (token, expert) pick goes through that
+    expert's MLP alone, products rounded to the tensor dtype, fp32 sum rounded once, plus the shared expert."""
+    k = idx.shape[1]
+    scale = out.float().abs().max().item()
+    cache = {}
+
+    def expert_w(e):
+        if e not in cache:
+            ex = moe.local_experts[e]
+            cache[e] = tuple(t.weight.detach().cpu() for t in (ex.gate_proj, ex.up_proj, ex.down_proj))
+        return cache[e]
+
+    shared = None
+    if moe.shared_expert is not None:
+        s = moe.shared_expert
+        shared = tuple(t.weight.detach().cpu() for t in (s.gate_proj, s.up_proj, s.down_proj))
+    worst = 0.0
+    for t in sample:
+        row = x_tokens[t : t + 1]
+        acc = torch.zeros(1, row.shape[1], dtype=torch.float32)
+        for j in range(k):
+            if keep is not None and not bool(keep[t * k + j]):
+                continue
+            y = O.mlp(row, *expert_w(int(idx[t, j])))
+            acc += (y * wts[t, j]).float()
+        ref = acc.to(row.dtype)
+        if shared is not None:
+            ref = ref + O.mlp(row, *shared)
+        worst = max(worst, (out[t].float() - ref[0].float()).abs().max().item())
+    assert worst <= rtol * scale, (worst, scale)
+
+
+def test_mixtral_shape_forward_full_size(gpu):
+    """8192 tokens, hidden 4096, FFN 14336, 8 experts, top-2, bf16 (the grouped-GEMM benchmark shape): routing
+    bit-exact against the oracle on the same logits, permutation bit-exact, outputs of sampled tokens within 1e-2."""
+    import bench
+    from picotron_amd import _ops
+
+    w = bench.WORKLOADS["c3"]
+    moe = bench.build_layer(w, gpu, torch.bfloat16)
+    x = torch.randn(w["T"], w["H"], generator=torch.Generator().manual_seed(0)).bfloat16()
+    with torch.no_grad():
+        xg = x.to(gpu)
+        out = moe(xg.view(1, w["T"], w["H"])).view(w["T"], w["H"]).cpu()
+        logits = moe.gate(xg).cpu()
+        idx, wts = moe._route(xg)
+        plan = _ops.permute_plan(idx.reshape(-1), w["E"])
+    ridx, rw, _ = O.softmax_topk_route(logits, w["k"])
+    assert torch.equal(idx.cpu(), ridx)                                    # incl. the tie rows of bf16 logits
+    assert int(O.tie_rows(logits, w["k"]).sum()) > 0
+    order, inv, counts = O.permute_plan_fast(ridx.reshape(-1), w["E"])
+    assert torch.equal(plan.order.cpu().long(), order) and torch.equal(plan.counts.cpu(), counts)
+    _sample_check(moe, x, out, ridx, wts.cpu(), None, range(0, w["T"], w["T"] // 24), rtol=1e-2)
+
+
+def test_fine_grained_skewed_capacity_full_size(gpu):
+    """16384 tokens, hidden 2048, 64 experts of FFN 1408, top-6, shared expert 2816, Zipf(1.1) router bias,
+    capacity factor 1.25 with drops: drop set bit-exact, outputs of sampled tokens within 1e-2."""
+    import bench
+    from picotron_amd import _ops
+    from picotron_amd.expert_parallel.capacity_moe import compute_capacity
+
+    w = bench.WORKLOADS["c4"]
+    moe = bench.build_layer(w, gpu, torch.bfloat16)
+    x = torch.randn(w["T"], w["H"], generator=torch.Generator().manual_seed(0)).bfloat16()
+    with torch.no_grad():
+        xg = x.to(gpu)
+        out = moe(xg.view(1, w["T"], w["H"])).view(w["T"], w["H"]).cpu()
+        logits = moe.gate(xg).cpu()
+        idx, wts = moe._route(xg)
+    ridx, rw, _ = O.softmax_topk_route(logits, w["k"])
+    ties = O.tie_rows(logits, w["k"])
+    assert torch.equal(idx.cpu(), ridx)
+    C = compute_capacity(w["T"], w["k"], w["E"], w["cap"])
+    assert C == 1920
+    within, counts = O.slot_assignment(ridx.reshape(-1), w["E"])
+    keep = within < C
+    plan = _ops.permute_plan(idx.reshape(-1), w["E"], capacity=C)
+    assert torch.equal(plan.inv_order.cpu() >= 0, keep)                    # the drop set
+    assert 0 < int((~keep).sum()) < keep.numel() and int(counts.max()) > C  # the skew really overflows experts
+    assert torch.equal(plan.kept_counts.cpu(), counts.clamp(max=C))
+    sample = list(range(0, w["T"], w["T"] // 24))
+    dropped_tokens = torch.nonzero((~keep).view(-1, w["k"]).any(1)).squeeze(1)[:8].tolist()
+    _sample_check(moe, x, out, ridx, wts.cpu(), keep, sample + dropped_tokens, rtol=1e-2)
+    assert int(ties.sum()) >= 0
