@@ -227,6 +227,9 @@ def main():
     ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-times", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="after the timed steps also launch a plain 1 GiB copy kernel three times: the known-size "
+                         "reference that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU (the EP=1 MoE hot path); run with --gpus 1")
@@ -277,6 +280,13 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     timer.enabled = False
+    if args.traffic_probe:
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)  # 1 GiB read + 1 GiB written per launch
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.neg(src, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     tokens_per_s = w["T"] / (ms_per_step * 1e-3)
     log(f"[bench] {args.workload}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tokens/s")
 

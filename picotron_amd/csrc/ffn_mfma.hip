@@ -34,6 +34,12 @@ constexpr int kNumXcd = 8;
 #define PICOMOE_MFMA_WAVES 8
 #endif
 constexpr int kWaves = PICOMOE_MFMA_WAVES;
+#ifndef PICOMOE_PREFETCH_FWD
+#define PICOMOE_PREFETCH_FWD 0
+#endif
+#ifndef PICOMOE_PREFETCH_BWD
+#define PICOMOE_PREFETCH_BWD 4
+#endif
 
 enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
 
@@ -64,9 +70,10 @@ struct MfmaParams {
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
 };
 
-__device__ __forceinline__ int swz(int row) {
-    return (row + (row >> 3)) & 7;
-}
+// K-major tiles: 16-byte chunk swizzle of tile row `row`.  A ds_read_b128 serves 16 lanes (16 consecutive rows, one
+// chunk each) per cycle; rows are 128 B, half the 256 B bank span, so rows 2i and 2i+1 cover all banks between them
+// and (row >> 1) & 7 puts the 8 row pairs on 8 different chunks: no bank conflicts (measured: 4 cycles per read).
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 // X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
 __device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
 
@@ -84,6 +91,9 @@ __device__ __forceinline__ s16x4_t lds_read_tr(const char* p) {
 struct TileCoord {
     int e, n_tile, m_tile, rows;  // rows: valid M rows (M-grouped) or valid K rows (wgrad)
     int64_t row0;                 // first row of the tile (M-grouped) or of the expert segment (wgrad)
+    // L2 prefetch shares: of the tiles one XCD runs at a time, a_sn share this tile's A slices and b_sn its B slices;
+    // this tile touches lines a_si, a_si + a_sn, ... of an A slice and b_si, b_si + b_sn, ... of a B slice
+    int a_si, a_sn, b_si, b_sn;
 };
 
 // Logical tile id of this block with the XCD remap, or -1.
@@ -136,6 +146,10 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
             tc->row0 = start + (int64_t)m * BM;
             const int64_t left = c - (int64_t)m * BM;
             tc->rows = left < BM ? (int)left : BM;
+            tc->a_sn = n_tiles < 4 ? n_tiles : 4;
+            tc->a_si = tc->n_tile % tc->a_sn;
+            tc->b_sn = me < 8 ? (int)me : 8;
+            tc->b_si = m % tc->b_sn;
             return true;
         }
         L -= te;
@@ -144,15 +158,27 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
     return false;
 }
 
+// wgrad tiles: expert by expert; inside an expert the P x Q tile grid is walked in bands of 4 tile columns and, inside
+// a band, in groups of 8 tile rows (tile row fastest inside a group), so that any 32 consecutive tiles -- what one
+// XCD's 32 CUs run at a time -- form an 8 x 4 patch that needs only 8 + 4 operand slices per k-step from its L2.
 __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, TileCoord* tc) {
     const int64_t per_e = (int64_t)m_tiles * n_tiles;
     const int64_t L = logical_tile(per_e * E);
     if (L < 0) return false;
     const int e = (int)(L / per_e);
-    const int64_t rem = L % per_e;
+    const int rem = (int)(L % per_e);
+    constexpr int GM = 8, GN = 4;
+    const int band = rem / (m_tiles * GN), r = rem % (m_tiles * GN);
+    const int wn = n_tiles - band * GN < GN ? n_tiles - band * GN : GN;
+    const int g = r / (GM * wn), r2 = r % (GM * wn);
+    const int hm = m_tiles - g * GM < GM ? m_tiles - g * GM : GM;
     tc->e = e;
-    tc->n_tile = (int)(rem / m_tiles);
-    tc->m_tile = (int)(rem % m_tiles);
+    tc->m_tile = g * GM + r2 % hm;
+    tc->n_tile = band * GN + r2 / hm;
+    tc->a_sn = wn;
+    tc->a_si = r2 / hm;
+    tc->b_sn = hm;
+    tc->b_si = r2 % hm;
     int64_t start = 0;
     for (int i = 0; i < e; ++i) start += counts[i];
     tc->row0 = start;
@@ -264,8 +290,69 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         const int kr = kt * BK + wave * KPW + q * 2 + (lane >> 5);
         return kr < tc.rows ? 0 : tc.rows - 1 - kr;
     };
-    // `full` (a std::bool_constant): the tile has all 256 rows, so the per-wave / per-row checks vanish at compile time
-    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq, auto /*full*/) {
+    // ------------------------------------------------------------------------------------------
+    // L2 prefetch.  The demand loads of the blocks that share an operand slice reach the L2 together, and when the
+    // slice still has to come from HBM they all queue behind the same misses.  So every k-step each wave touches
+    // (one 4-byte load per 64 bytes into a scratch register nobody reads) its share of the lines of a slice
+    // kPrefetchDist k-steps ahead: the first half of the waves lines of the A slice, the second half lines of the B
+    // slice.
+    // ------------------------------------------------------------------------------------------
+    constexpr int kPrefetchDist = T::kBKMajor ? PICOMOE_PREFETCH_FWD : PICOMOE_PREFETCH_BWD;
+    const char* pf_ptr;   // this lane's line at k-tile 0
+    int64_t pf_step;      // bytes per k-tile
+    {
+        const bool pf_b = wave >= NW / 2;
+        const int q = (wave % (NW / 2)) * 64 + lane, half = q & 1;
+        const int si = pf_b ? tc.b_si : tc.a_si, sn = pf_b ? tc.b_sn : tc.a_sn;
+        int j = si + sn * (q >> 1);  // line of the 256-line slice
+        if (j >= 256) j = si;
+        // X-major slices: line j is 128 bytes of k row j / 4; a segment shorter than one k-tile clamps the row
+        int kr = j >> 2;
+        if (MODE == kWgrad && kr >= tc.rows) kr = tc.rows > 0 ? tc.rows - 1 : 0;
+        if (!pf_b) {
+            pf_step = a_step;
+            if (T::kAKMajor) {
+                const int r = j < tc.rows ? j : tc.rows - 1;
+                pf_ptr = (const char*)(p.A + (tc.row0 + r) * p.lda) + half * 64;
+            } else {
+                int64_t col = (int64_t)tc.m_tile * BM + (j & 3) * 64 + half * 32;
+                col = col + 8 <= p.M ? col : p.M - 8;
+                pf_ptr = (const char*)(p.A + (tc.row0 + kr) * p.lda + col);
+            }
+        } else {
+            pf_step = b_step;
+            if (MODE == kGateUp) {
+                const uint16_t* m = j < 128 ? p.B0 : p.B1;
+                pf_ptr = (const char*)(m + (int64_t)tc.e * p.b_expert_stride + ((int64_t)tc.n_tile * 128 + (j & 127)) * p.ldb) + half * 64;
+            } else if (MODE == kDown) {
+                pf_ptr = (const char*)(p.B0 + (int64_t)tc.e * p.b_expert_stride + ((int64_t)tc.n_tile * BN + j) * p.ldb) + half * 64;
+            } else {
+                int64_t col = (int64_t)tc.n_tile * BN + (j & 3) * 64 + half * 32;
+                col = col + 8 <= p.N ? col : p.N - 8;
+                const uint16_t* m = MODE == kWgrad ? p.B0 + tc.row0 * p.ldb : p.B0 + (int64_t)tc.e * p.b_expert_stride;
+                pf_ptr = (const char*)(m + (int64_t)kr * p.ldb + col);
+            }
+        }
+    }
+    const int64_t pf_switch_delta = wave >= NW / 2 ? b_switch_delta : 0;
+    // wgrad: only k-tiles that lie completely inside the expert's rows are prefetched
+    const int pf_n_kt = MODE == kWgrad ? tc.rows / BK : n_kt;
+    // the lane's pointer moves on by one k-tile per call until it reaches the last k-tile that may be touched
+    const int pf_kt0 = kPrefetchDist < pf_n_kt ? kPrefetchDist : (pf_n_kt > 0 ? pf_n_kt - 1 : 0);
+    const char* pf_cur = pf_ptr + (int64_t)pf_kt0 * pf_step + (pf_kt0 >= b_switch_kt ? pf_switch_delta : 0);
+    auto prefetch_l2 = [&](int kt) {
+        if (kPrefetchDist == 0) return;
+        // Destination v255: a register the kernel never allocates (it needs fewer than 255; the build checks the
+        // generated code for any other mention of v255), so a load still in flight cannot land on a live value.
+        asm volatile("global_load_dword v255, %0, off" ::"v"(pf_cur) : "v255", "memory");
+        const int kp = kt + kPrefetchDist + 1;  // the k-tile of the next call
+        int64_t adv = kp < pf_n_kt ? pf_step : 0;
+        if (MODE == kDgradX && kp == b_switch_kt) adv += pf_switch_delta;
+        pf_cur += adv;
+    };
+
+    // `active` (a std::bool_constant): false in the loop copy of the waves that only load and synchronise
+    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq, auto /*active*/) {
         char* base = lds + stage * kStageBytes;
         const char* ab = a_base + (int64_t)kt * a_step;
         const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
@@ -283,8 +370,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     };
     // half of a wave's loads for one tile: part 0 or 1
-    auto issue_loads_part = [&](int kt, int stage, int part, auto full) {
-        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{}, full);
+    auto issue_loads_part = [&](int kt, int stage, int part, auto active) {
+        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{}, active);
     };
 
     // ------------------------------------------------------------------------------------------
@@ -344,8 +431,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         return __builtin_bit_cast(bf16x8_t, v);
     };
     // reads the fragments of k sub-step kk from the stage the address registers currently point at
-    auto read_frags = [&](int kk, int buf, auto full) {
-        if (!decltype(full)::value && !wave_active) return;
+    auto read_frags = [&](int kk, int buf, auto active) {
+        if (!decltype(active)::value) return;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             if (T::kAKMajor)
@@ -378,8 +465,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) zero_tail(bfr[buf][j]);
     };
-    auto mma = [&](int buf, auto full) {
-        if (!decltype(full)::value && !wave_active) return;
+    auto mma = [&](int buf, auto active) {
+        if (!decltype(active)::value) return;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -418,9 +505,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        read_frags(0, 0, std::false_type{});
+        if (wave_active) read_frags(0, 0, std::true_type{});
     }
-    auto k_loop = [&](auto full) {
+    auto k_loop = [&](auto active) {
     for (int kt = 0; kt < n_kt; ++kt) {
         const int stage = kt & 1;
         const bool tail = MODE == kWgrad && kt == n_kt - 1;
@@ -428,37 +515,41 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         // second half of the refill begun in the previous k-step.  Issued unconditionally (past the end the tile
         // index is clamped and the data land in a stage nobody reads) so that the loads sit in the same basic
         // block as the MFMAs and can be interleaved with them.
-        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1, full);
+        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1, active);
         if (tail) mask_tail(kt, 0, 0);
-        read_frags(1, 1, full);
-        mma(0, full);
+        read_frags(1, 1, active);
+        mma(0, active);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
+        prefetch_l2(kt);
         if (tail) mask_tail(kt, 1, 1);
-        read_frags(2, 0, full);
-        mma(1, full);
-        PICOMOE_INTERLEAVE(false)
+        read_frags(2, 0, active);
+        mma(1, active);
+        PICOMOE_INTERLEAVE(kPrefetchDist > 0)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 2, 0);
-        read_frags(3, 1, full);
-        mma(0, full);
+        read_frags(3, 1, active);
+        mma(0, active);
         PICOMOE_INTERLEAVE(false)
         __builtin_amdgcn_sched_barrier(0);
         // Every wave holds its last fragments of this stage in registers and the next tile has landed:
         // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        // all operand loads have landed; this k-step's prefetch load, the youngest in the queue, may stay in flight
+        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+        else __builtin_amdgcn_s_waitcnt(0x0F71);
         __syncthreads();
-        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0, full);
+        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0, active);
         if (tail) mask_tail(kt, 3, 1);
         flip_stage();
-        read_frags(0, 0, full);  // past the last tile this reads a stage that is not used any more
-        mma(1, full);
+        read_frags(0, 0, active);  // past the last tile this reads a stage that is not used any more
+        mma(1, active);
         PICOMOE_INTERLEAVE(true)
         __builtin_amdgcn_sched_barrier(0);
     }
     };
-    // two copies of the loop: full tiles (the common case) run without any per-wave checks
-    if (MODE == kWgrad || tc.rows >= BM) k_loop(std::true_type{});
+    // Two copies of the loop, picked per wave: waves that own rows of the tile run all of it; a wave whose 128 rows lie
+    // past the end of a short tail only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).
+    if (wave_active) k_loop(std::true_type{});
     else k_loop(std::false_type{});
 #undef PICOMOE_INTERLEAVE
     // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
