@@ -171,6 +171,58 @@ def fp8_quant_bandwidth(device, n=16384, h=4096, sets=6, iters=60):
     return nbytes / tq / 1e6, nbytes / td / 1e6, tq * 1e3, td * 1e3
 
 
+def fp8_gemm_variant(moe, step, w, steps):
+    """The same layer step with the forward gate/up GEMM on FP8 MFMA (E4M3 dispatch codes x per-row quantised weights,
+    re-quantised every step as in training): step time, and the FP8 kernel and the weight quantiser timed with events."""
+    import torch
+
+    from picotron_amd.expert_parallel import megakernel as mk
+
+    times = {"gate_up_fp8": [], "quantize_weights": []}
+    pool = [torch.cuda.Event(enable_timing=True) for _ in range(2 * 3 * steps + 8)]
+    state = {"on": False}
+
+    def wrap(name, fn):
+        def timed(*a, **kw):
+            if not state["on"] or len(pool) < 2:
+                return fn(*a, **kw)
+            st, en = pool.pop(), pool.pop()
+            st.record()
+            out = fn(*a, **kw)
+            en.record()
+            times[name].append((st, en))
+            return out
+        return timed
+
+    orig = (mk._gate_up_fp8, mk.quantize_expert_weights)
+    mk._gate_up_fp8 = wrap("gate_up_fp8", mk._gate_up_fp8)
+    mk.quantize_expert_weights = wrap("quantize_weights", mk.quantize_expert_weights)
+    moe.ep_fp8_gemm = True
+    try:
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        state["on"] = True
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        state["on"] = False
+        moe.ep_fp8_gemm = False
+        mk._gate_up_fp8, mk.quantize_expert_weights = orig
+    k_ms = sum(a.elapsed_time(b) for a, b in times["gate_up_fp8"]) / max(len(times["gate_up_fp8"]), 1)
+    q_ms = sum(a.elapsed_time(b) for a, b in times["quantize_weights"]) / max(steps, 1)  # two calls (gate, up) per step
+    flop = 4.0 * w["T"] * w["k"] * w["H"] * w["I"]
+    log(f"[bench] fp8 gate/up GEMM variant: {ms:.3f} ms/step, gate_up_fp8 {k_ms:.2f} ms ({flop / k_ms / 1e9:.0f} TFLOP/s), "
+        f"weight quantisation {q_ms:.2f} ms/step")
+    return {"ms_per_step": ms, "tokens_per_s": w["T"] / (ms * 1e-3), "gate_up_fp8_ms": k_ms,
+            "gate_up_fp8_tflops": flop / k_ms / 1e9, "frac_fp8_mfma_peak": flop / k_ms / 1e9 / 5000.0,
+            "weight_quant_ms_per_step": q_ms,
+            "note": "forward gate/up on v_mfma_f32_32x32x64_f8f6f4; down, dgrad and wgrad stay bf16; not the headline value"}
+
+
 def cpu_baseline(w, moe, budget_s=25.0):
     """The CPU oracle (port of the reference's naive torch path) on this box's host cores, on a token-subsampled
     batch of the same layer shape (same H / I / E / k and the same weights)."""
@@ -332,6 +384,9 @@ def main():
                                "dequant_frac_hbm": dg / HBM_PEAK_GBPS, "dequant_us": td,
                                "shape": "16384 x 4096 bf16 -> e4m3 + fp32 scale, 201392128 B per pass"}
         log(f"[bench] fp8 quant {qg:.0f} GB/s ({tq:.1f} us), dequant {dg:.0f} GB/s ({td:.1f} us)")
+
+    if w["fp8"] and not args.no_kernel_times:
+        result["fp8_gemm"] = fp8_gemm_variant(moe, step, w, args.steps)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, moe)

@@ -116,6 +116,15 @@ int picomoe_combine_bwd(const void* d_out, const void* y, const int32_t* inv_ord
 int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                         int64_t inter, const void* gate_w, const void* up_w, int dtype, void* act, void* inter13,
                         void* stream);
+/* The same gate||up GEMM + silu_and_mul on FP8 MFMA, fed by the FP8 dispatch: xq [n_rows, hidden] E4M3 codes with one
+ * fp32 scale per row (what _per_token_quant_fp8 ships, EP/ep_communications.py:63-68, instead of the dequantised rows
+ * of :100), gate_wq / up_wq [E, inter, hidden] codes with one fp32 scale per output row ([E * inter], quantised the
+ * same way, e.g. with picomoe_fp8_quant on the [E * inter, hidden] view).  g = (xq . gate_wq[e]^T) * x_scale * scale,
+ * fp32 accumulation; act / inter13 in bf16.  hidden % 256 == 0 and inter % 128 == 0, else PICOMOE_ERR_ARG.  The
+ * reference has no FP8 GEMM: results are compared with the bf16 GEMM on the dequantised rows at rtol 5e-2. */
+int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, const int64_t* counts, int num_experts, int64_t n_rows,
+                            int64_t hidden, int64_t inter, const void* gate_wq, const void* up_wq, const float* gate_scale,
+                            const float* up_scale, void* act, void* inter13, void* stream);
 /* Replaces the down grouped GEMM with its optional row-weight epilogue (EP/megakernel.py:305, :95-96). */
 int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden, int64_t inter,
                      const void* down_w, const void* row_weight, int dtype, void* y, void* stream);

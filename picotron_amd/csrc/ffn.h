@@ -41,6 +41,11 @@ int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_
 int ffn_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, int64_t P, int64_t Q,
                    void* out, hipStream_t st);
 
+// FP8 (E4M3) MFMA gate/up: codes + one fp32 scale per activation row and per weight row (ffn_fp8.hip)
+bool ffn_fp8_supported(const FfnShape& s);
+int ffn_fp8_gate_up(const FfnShape& s, const void* xq, const float* x_scale, const void* gq, const void* uq,
+                    const float* g_scale, const float* u_scale, void* act, void* inter13, hipStream_t st);
+
 // SwiGLU pieces shared by both families (fp32 arithmetic on values already rounded to the storage type).
 __device__ __forceinline__ float sigmoid_f32(float g) { return 1.0f / (1.0f + expf(-g)); }
 __device__ __forceinline__ float sigmoid_fast(float g) { return __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }

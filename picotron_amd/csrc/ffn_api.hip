@@ -22,6 +22,18 @@ extern "C" int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num
     return ffn_simple_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
 }
 
+extern "C" int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, const int64_t* counts, int num_experts,
+                                       int64_t n_rows, int64_t hidden, int64_t inter, const void* gate_wq, const void* up_wq,
+                                       const float* gate_scale, const float* up_scale, void* act, void* inter13,
+                                       void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, PICOMOE_BF16));
+    PICOMOE_CHECK_ARG(ffn_fp8_supported(s));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(xq && x_scale && gate_wq && up_wq && gate_scale && up_scale && act);
+    return ffn_fp8_gate_up(s, xq, x_scale, gate_wq, up_wq, gate_scale, up_scale, act, inter13, (hipStream_t)stream);
+}
+
 extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                                 int64_t inter, const void* down_w, const void* row_weight, int dtype, void* y, void* stream) {
     FfnShape s;

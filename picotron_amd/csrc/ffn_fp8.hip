@@ -1,0 +1,245 @@
+// FP8 (E4M3) MFMA kernel for the gate/up projection of the expert FFN on gfx950 (MI355X): the per-token quantised
+// activations of the FP8 dispatch (codes + one fp32 scale per row) meet expert weights quantised the same way
+// (one scale per output row) in v_mfma_f32_32x32x64_f8f6f4, fp32 accumulation, and the two scales are applied to
+// the accumulators in the epilogue, fused with SwiGLU.
+//
+// Same frame as the bf16 kernels: 256 x 256 block tile, 8 wavefronts (two per SIMD) of 128 x 64, two 64 KB LDS
+// stages filled by 16-byte direct-to-LDS loads.  A 128-byte LDS row now holds 128 k values, so one k-step is two
+// MFMA sub-steps of K = 64 and a tile needs half as many k-steps, loads and barriers per FLOP.  A lane feeds an MFMA
+// with 32 consecutive k bytes of its row (two ds_read_b128); which 32 of the 64 go to which lane half is free as
+// long as both operands agree, because the instruction only sums over k.
+#include <type_traits>
+
+#include "ffn.h"
+#include "mfma_tiles.h"
+
+namespace {
+
+constexpr int kFp8Waves = 8;
+constexpr int kFp8BK = 128;  // k values (bytes) per k-step
+
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
+struct Fp8Params {
+    const int64_t* counts;
+    int E;
+    int64_t n_rows, H, I;
+    int n_tiles;
+    const uint8_t* xq;     // [n_rows, H] e4m3 codes
+    const float* x_scale;  // [n_rows]
+    const uint8_t* gq;     // [E, I, H]
+    const uint8_t* uq;
+    const float* g_scale;  // [E * I]
+    const float* u_scale;
+    uint16_t* act;      // [n_rows, I] bf16
+    uint16_t* inter13;  // [n_rows, 2I] bf16 or null
+};
+
+__global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8Params p) {
+    constexpr int NI = 4, NJ = 2, kWaveCols = 4, CW = 64, QN = 4, RPW = 32;
+    __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
+    TileCoord tc;
+    if (!locate_m_grouped(p.counts, p.E, p.n_tiles, &tc)) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / kWaveCols, wn = wave % kWaveCols;
+    const int l31 = lane & 31, hi = lane >> 5;
+    const int n_kt = (int)(p.H / kFp8BK);
+    const bool wave_active = wm * 128 < tc.rows;
+
+    // global -> LDS: wave w fills rows [32w, 32w + 32) of both tiles, 8 rows (128 B each) per instruction.  B tile:
+    // per wave column (64 rows) 32 gate rows then 32 up rows of the same FFN columns: even waves load gate rows.
+    uint32_t a_off[QN], b_off[QN];
+    const char* a_base = (const char*)(p.xq + tc.row0 * p.H);
+    const uint8_t* bmat = (wave & 1) ? p.uq : p.gq;
+    const char* b_base = (const char*)(bmat + ((int64_t)tc.e * p.I + (int64_t)tc.n_tile * 128 + (wave >> 1) * 32) * p.H);
+#pragma unroll
+    for (int q = 0; q < QN; ++q) {
+        const int r = wave * RPW + q * 8 + (lane >> 3);
+        const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the segment re-read its last row (never stored)
+        a_off[q] = (uint32_t)(ar * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
+        b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
+    }
+    auto issue_loads = [&](int kt, int stage, int q0) {  // half of a wave's loads for one k-tile
+        char* base = lds + stage * kStageBytes;
+        const char* ab = a_base + (int64_t)kt * kFp8BK;
+        const char* bb = b_base + (int64_t)kt * kFp8BK;
+#pragma unroll
+        for (int q = q0; q < q0 + QN / 2; ++q) {
+            load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
+            load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * RPW + q * 8) * 128);
+        }
+    };
+
+    // LDS -> fragments.  Lane (row l & 31, half l >> 5) of sub-step s reads the 16-byte chunks 4s + 2*half and
+    // 4s + 2*half + 1 of its row; with the XOR swizzle those are the address of chunk 2*half XOR (s << 6) and XOR 16.
+    uint32_t a_ad[NI], b_ad[NJ];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int ra = wm * 128 + i * 32 + l31;
+        a_ad[i] = lds0 + ra * 128 + (((2 * hi) ^ swz(ra)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int rb = wn * CW + j * 32 + l31;
+        b_ad[j] = lds0 + kTileBytes + rb * 128 + (((2 * hi) ^ swz(rb)) << 4);
+    }
+    auto flip_stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) a_ad[i] ^= (uint32_t)kStageBytes;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) b_ad[j] ^= (uint32_t)kStageBytes;
+    };
+    auto read_frag = [&](uint32_t ad, int s) -> i32x8_t {
+        const u32x4_t lo = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)(ad ^ (uint32_t)(s << 6));
+        const u32x4_t up = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)(ad ^ (uint32_t)(s << 6) ^ 16u);
+        i32x8_t v;
+        v[0] = (int)lo[0]; v[1] = (int)lo[1]; v[2] = (int)lo[2]; v[3] = (int)lo[3];
+        v[4] = (int)up[0]; v[5] = (int)up[1]; v[6] = (int)up[2]; v[7] = (int)up[3];
+        return v;
+    };
+
+    f32x16_t acc[NI][NJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    i32x8_t af[2][NI], bfr[2][NJ];
+    auto read_frags = [&](int s, int buf, auto active) {
+        if (!decltype(active)::value) return;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) af[buf][i] = read_frag(a_ad[i], s);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) bfr[buf][j] = read_frag(b_ad[j], s);
+    };
+    auto mma = [&](int buf, auto active) {
+        if (!decltype(active)::value) return;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    };
+    // one sub-step: 8 MFMAs (64 cycles each), the 12 LDS reads of the next sub-step and 4 direct-to-LDS loads,
+    // spread one MFMA : two reads : one load over the first MFMAs
+#define PICOMOE_FP8_INTERLEAVE()                                  \
+    _Pragma("unroll") for (int s_ = 0; s_ < 6; ++s_) {            \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);        \
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
+    }                                                             \
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+
+    if (n_kt > 0) {
+        issue_loads(0, 0, 0);
+        issue_loads(0, 0, QN / 2);
+        if (n_kt > 1) {
+            issue_loads(1, 1, 0);
+            issue_loads(1, 1, QN / 2);
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): tile 0 has landed, tile 1 may still be in flight
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();
+        if (wave_active) read_frags(0, 0, std::true_type{});
+    }
+    auto k_loop = [&](auto active) {
+        for (int kt = 0; kt < n_kt; ++kt) {
+            const int stage = kt & 1;
+            __builtin_amdgcn_sched_barrier(0);
+            // second half of the refill begun in the previous k-step (clamped past the end: lands in a dead stage)
+            issue_loads(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, QN / 2);
+            read_frags(1, 1, active);
+            mma(0, active);
+            PICOMOE_FP8_INTERLEAVE()
+            __builtin_amdgcn_sched_barrier(0);
+            // every wave holds its last fragments of this stage in registers and the next tile has landed
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            issue_loads(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0);
+            flip_stage();
+            read_frags(0, 0, active);  // past the last tile this reads a stage that is not used any more
+            mma(1, active);
+            PICOMOE_FP8_INTERLEAVE()
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (wave_active) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
+#undef PICOMOE_FP8_INTERLEAVE
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    // epilogue: scale, round g and u to bf16 (what the two Linear outputs of the reference hold), SwiGLU, and stage
+    // 32 rows at a time through a wave-private slice of LDS so that the stores are 16-byte lanes of contiguous rows
+    float* row_scale = (float*)(lds + kStageBytes);  // 256 floats, past the staging slices
+    if (tid < BM) row_scale[tid] = p.x_scale[tc.row0 + (tid < tc.rows ? tid : tc.rows - 1)];
+    const int64_t I = p.I;
+    const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
+    const float gs = p.g_scale[(int64_t)tc.e * I + col0 + l31], us = p.u_scale[(int64_t)tc.e * I + col0 + l31];
+    __syncthreads();
+    constexpr int kEpiCols = CW / 2;
+    constexpr int kEpiStride = (kEpiCols + 8) * 2;
+    char* epi = lds + wave * (32 * kEpiStride);
+    constexpr int kChunksPerRow = kEpiCols / 8;
+    constexpr int kReadIters = 32 * kChunksPerRow / 64;
+    auto stage_block = [&](auto value) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
+            *(uint16_t*)(epi + row * kEpiStride + l31 * 2) = (uint16_t)f32_to_bf16_bits(value(r));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    auto for_chunks = [&](int i, auto f) {
+#pragma unroll
+        for (int it = 0; it < kReadIters; ++it) {
+            const int idx = it * 64 + lane;
+            const int row = idx / kChunksPerRow, ch = idx % kChunksPerRow;
+            const u32x4_t v = *(const u32x4_t*)(epi + row * kEpiStride + ch * 16);
+            const int trow = wm * 128 + i * 32 + row;
+            if (trow < tc.rows) f(trow, ch * 8, v);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float sx = row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)];
+            acc[i][0][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][r] * sx * gs));
+            acc[i][1][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][r] * sx * us));
+        }
+        stage_block([&](int r) {
+            const float g = acc[i][0][r], u = acc[i][1][r];
+            return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
+        });
+        for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.act + (tc.row0 + trow) * I + col0 + c) = v; });
+        if (p.inter13) {
+            stage_block([&](int r) { return acc[i][0][r]; });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + col0 + c) = v; });
+            stage_block([&](int r) { return acc[i][1][r]; });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + I + col0 + c) = v; });
+        }
+    }
+}
+
+}  // namespace
+
+bool ffn_fp8_supported(const FfnShape& s) { return s.H % 256 == 0 && s.I % 128 == 0 && s.H >= 256 && s.I >= 128; }
+
+int ffn_fp8_gate_up(const FfnShape& s, const void* xq, const float* x_scale, const void* gq, const void* uq,
+                    const float* g_scale, const float* u_scale, void* act, void* inter13, hipStream_t st) {
+    Fp8Params p{};
+    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.H = s.H; p.I = s.I; p.n_tiles = (int)(s.I / 128);
+    p.xq = (const uint8_t*)xq; p.x_scale = x_scale;
+    p.gq = (const uint8_t*)gq; p.uq = (const uint8_t*)uq; p.g_scale = g_scale; p.u_scale = u_scale;
+    p.act = (uint16_t*)act; p.inter13 = (uint16_t*)inter13;
+    hipLaunchKernelGGL(ffn_fp8_gate_up_kernel, dim3(grid_m_grouped(s, p.n_tiles)), dim3(kFp8Waves * 64), 0, st, p);
+    return picomoe_launch_status();
+}

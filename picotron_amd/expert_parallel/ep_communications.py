@@ -50,12 +50,16 @@ class _Fp8RoundTrip(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x):
         q, scale = _per_token_quant_fp8(x)
-        return _dequant_fp8(q, scale, x.dtype)
+        ctx.mark_non_differentiable(q, scale)
+        return _dequant_fp8(q, scale, x.dtype), q, scale
 
     @staticmethod
-    def backward(ctx, grad_out):
+    def backward(ctx, grad_out, _grad_q, _grad_scale):
         return grad_out
 
 
-def fp8_round_trip(x):
-    return _Fp8RoundTrip.apply(x)
+def fp8_round_trip(x, with_codes=False):
+    """dequantise(quantise(x)) with a straight-through gradient; ``with_codes`` also returns the E4M3 codes and the
+    per-row scales the dequantised rows were built from (for the FP8 GEMM)."""
+    out, q, scale = _Fp8RoundTrip.apply(x)
+    return (out, q, scale) if with_codes else out

@@ -81,6 +81,10 @@ class MoELayer(nn.Module):
         self.ep_num_tiles = getattr(config, "ep_num_tiles", 1)
         self.ep_backend = getattr(config, "ep_backend", "torch")
         self.ep_fp8_dispatch = getattr(config, "ep_fp8_dispatch", False)
+        # not in the reference: with the FP8 dispatch on, feed the forward gate/up GEMM with the E4M3 codes on FP8 MFMA
+        # (weights quantised per output row) instead of the dequantised rows on bf16 MFMA
+        self.ep_fp8_gemm = getattr(config, "ep_fp8_gemm", False)
+        self._fp8_weights = None
 
         self.ep_capacity_factor = getattr(config, "ep_capacity_factor", 0.0)
         self.ep_capacity_dropless = getattr(config, "ep_capacity_dropless", True)
@@ -195,13 +199,21 @@ class MoELayer(nn.Module):
         num_tokens = tokens.shape[0]
         shared = self._shared_start(tokens)
         latent = self._maybe_down(tokens)
-        if self.ep_fp8_dispatch:
-            # one quantise -> dequantise per token equals one per routed row (a row op on identical rows)
-            latent = fp8_round_trip(latent)
         n_rows = num_tokens * self.top_k
         plan = _ops.permute_plan(topk_idx.reshape(-1), self.num_local_experts)
+        codes = None
+        if self.ep_fp8_dispatch:
+            # one quantise -> dequantise per token equals one per routed row (a row op on identical rows)
+            if self._use_fp8_gemm(latent):
+                latent, q, scale = fp8_round_trip(latent, with_codes=True)
+                # the codes travel like the rows: gathered into expert order (two codes per 16-bit element)
+                q16 = q.view(torch.uint8).view(torch.int16).view(torch.bfloat16)
+                src = torch.div(plan.order, self.top_k, rounding_mode="floor")
+                codes = (_ops.gather_rows(q16, plan.order, self.top_k, n_rows).view(torch.uint8), scale[src])
+            else:
+                latent = fp8_round_trip(latent)
         x_sorted = _ops.expand_permute(latent, plan.order, plan.inv_order, self.top_k, n_rows)
-        y_sorted = self._grouped_experts(x_sorted, plan.counts)
+        y_sorted = self._grouped_experts(x_sorted, plan.counts, codes)
         y = _ops.unpermute_combine(y_sorted, topk_weights, plan.inv_order, plan.order, num_tokens, self.top_k)
         return self._finalize(y, shared)
 
@@ -218,13 +230,37 @@ class MoELayer(nn.Module):
         )
         return self._finalize(y, shared)
 
-    def _grouped_experts(self, x_sorted, counts):
-        """Run the local experts on rows already grouped by expert; ``counts[e]`` rows go to expert ``e``."""
+    def _use_fp8_gemm(self, x):
+        return (self.ep_fp8_gemm and x.dtype == torch.bfloat16 and x.shape[0] > 0
+                and megakernel.fp8_gemm_supported(self.expert_dim, self.local_experts[0].gate_proj.weight.shape[0]))
+
+    def _quantized_weights(self):
+        """E4M3 codes + per-row scales of the stacked gate / up weights.  Training: redone every forward (the
+        optimizer changes the weights every step).  Eval: kept until a parameter's version counter moves; after a
+        write that bypasses the counters (``p.data``) call ``invalidate_fp8_weights``."""
+        gates, ups, _ = self._expert_params()
+        key = (self._stacks[0].data_ptr(), self._stacks[1].data_ptr(), tuple(p._version for p in gates + ups))
+        if self.training or self._fp8_weights is None or self._fp8_weights[0] != key:
+            with torch.no_grad():
+                gq, gs = megakernel.quantize_expert_weights(self._stacks[0])
+                uq, us = megakernel.quantize_expert_weights(self._stacks[1])
+            self._fp8_weights = (key, (gq, gs, uq, us))
+        return self._fp8_weights[1]
+
+    def invalidate_fp8_weights(self):
+        self._fp8_weights = None
+
+    def _grouped_experts(self, x_sorted, counts, codes=None):
+        """Run the local experts on rows already grouped by expert; ``counts[e]`` rows go to expert ``e``.
+        ``codes`` (optional): ``(E4M3 codes [N,H] uint8, scale [N])`` of the same rows for the FP8 gate/up GEMM."""
         if x_sorted.shape[0] == 0:
             return x_sorted
         _lib.require_cuda(x_sorted)
         gate_w, up_w, down_w = self._stacked_weights()
-        return megakernel.fused_moe(x_sorted, counts, gate_w, up_w, down_w)
+        fp8 = None
+        if codes is not None:
+            fp8 = (codes[0], codes[1]) + self._quantized_weights()
+        return megakernel.fused_moe(x_sorted, counts, gate_w, up_w, down_w, fp8=fp8)
 
     def _run_local_experts(self, x, local_expert_idx):
         """Run the local experts on ``x`` given each row's expert id, preserving the input order."""

@@ -55,6 +55,43 @@ def _gate_up(x, counts, gate_w, up_w, keep_inter13):
     return act, inter13
 
 
+def fp8_gemm_supported(hidden, inter):
+    """Shapes the FP8 MFMA gate/up kernel tiles (everything else runs the bf16 kernels on the dequantised rows)."""
+    return hidden % 256 == 0 and inter % 128 == 0
+
+
+def quantize_expert_weights(w):
+    """w [E, I, H] bf16/fp32 -> (E4M3 codes uint8 [E, I, H], fp32 scale [E * I]): every output row gets the scale
+    amax / 448 of the FP8 dispatch quantiser (``_per_token_quant_fp8``), with the same kernel."""
+    lib = _lib.load()
+    _lib.require_cuda(w)
+    w = w.contiguous()
+    E, I, H = w.shape
+    q = torch.empty((E, I, H), dtype=torch.uint8, device=w.device)
+    scale = torch.empty((E * I,), dtype=torch.float32, device=w.device)
+    _lib.check(
+        lib.picomoe_fp8_quant(_lib.ptr(w), _lib.dtype_code(w.dtype), E * I, H, _lib.ptr(q), _lib.ptr(scale), _lib.stream_ptr()),
+        "picomoe_fp8_quant",
+    )
+    return q, scale
+
+
+def _gate_up_fp8(xq, x_scale, counts, gate_q, gate_scale, up_q, up_scale, keep_inter13, dtype=torch.bfloat16):
+    """gate/up GEMM + SwiGLU on FP8 MFMA: xq [N,H] E4M3 codes + x_scale [N]; weights as ``quantize_expert_weights``."""
+    lib = _lib.load()
+    E, I, H = gate_q.shape
+    N = xq.shape[0]
+    act = torch.empty((N, I), dtype=dtype, device=xq.device)
+    inter13 = torch.empty((N, 2 * I), dtype=dtype, device=xq.device) if keep_inter13 else None
+    _lib.check(
+        lib.picomoe_ffn_gate_up_fp8(_lib.ptr(xq), _lib.ptr(x_scale), _lib.ptr(counts), E, N, H, I, _lib.ptr(gate_q),
+                                    _lib.ptr(up_q), _lib.ptr(gate_scale), _lib.ptr(up_scale), _lib.ptr(act),
+                                    _lib.ptr(inter13), _lib.stream_ptr()),
+        "picomoe_ffn_gate_up_fp8",
+    )
+    return act, inter13
+
+
 def _down(act, counts, down_w, row_weight):
     lib = _lib.load()
     E, H, I = down_w.shape
@@ -157,7 +194,7 @@ def fused_moe_backward(x_sorted, counts, gate_w, up_w, down_w, dy):
 
 class _FusedMoE(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x_sorted, gate_w, up_w, down_w, counts, row_weight):
+    def forward(ctx, x_sorted, gate_w, up_w, down_w, counts, row_weight, fp8=None):
         x, counts, (gw, uw, dw) = _prep(x_sorted, counts, gate_w, up_w, down_w)
         _check_weights(x, gw, uw, dw)
         ctx.counts = counts
@@ -168,7 +205,13 @@ class _FusedMoE(torch.autograd.Function):
             return torch.empty((0, x.shape[1]), device=x.device, dtype=x.dtype)
         ctx.empty = False
         needs_grad = any(ctx.needs_input_grad[:4]) or (ctx.has_rw and ctx.needs_input_grad[5])
-        act, inter13 = _gate_up(x, counts, gw, uw, keep_inter13=needs_grad)
+        if fp8 is not None:
+            # forward gate/up on FP8 MFMA from the dispatch's codes; the backward below is the bf16 one on x_sorted
+            xq, x_scale, gate_q, gate_scale, up_q, up_scale = fp8
+            act, inter13 = _gate_up_fp8(xq.contiguous(), x_scale.contiguous(), counts, gate_q, gate_scale, up_q, up_scale,
+                                        keep_inter13=needs_grad, dtype=x.dtype)
+        else:
+            act, inter13 = _gate_up(x, counts, gw, uw, keep_inter13=needs_grad)
         rw = row_weight.to(x.dtype).contiguous() if ctx.has_rw else None
         y = _down(act, counts, dw, rw)
         if needs_grad:
@@ -179,7 +222,7 @@ class _FusedMoE(torch.autograd.Function):
     def backward(ctx, grad_y):
         if ctx.empty:
             x, gw, uw, dw = ctx.saved_tensors
-            return torch.zeros_like(x), torch.zeros_like(gw), torch.zeros_like(uw), torch.zeros_like(dw), None, None
+            return torch.zeros_like(x), torch.zeros_like(gw), torch.zeros_like(uw), torch.zeros_like(dw), None, None, None
         x, gw, uw, dw, act, inter13, rw = ctx.saved_tensors
         counts = ctx.counts
         dy = grad_y.contiguous()
@@ -195,12 +238,16 @@ class _FusedMoE(torch.autograd.Function):
         d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device)
         d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
         d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
-        return dx, d_gate, d_up, d_down, None, d_rw
+        return dx, d_gate, d_up, d_down, None, d_rw, None
 
 
-def fused_moe(x_sorted, counts, gate_w, up_w, down_w, row_weight=None):
-    """Differentiable fused MoE expert FFN.  counts [E] = per-expert row counts."""
-    return _FusedMoE.apply(x_sorted, gate_w, up_w, down_w, counts, row_weight)
+def fused_moe(x_sorted, counts, gate_w, up_w, down_w, row_weight=None, fp8=None):
+    """Differentiable fused MoE expert FFN.  counts [E] = per-expert row counts.
+
+    ``fp8`` (optional, not in the reference): ``(xq [N,H] E4M3 codes, x_scale [N], gate_q, gate_scale, up_q,
+    up_scale)`` -- the rows of ``x_sorted`` as the FP8 dispatch ships them and the weights from
+    ``quantize_expert_weights``; the forward gate/up GEMM then runs on FP8 MFMA, everything else as without it."""
+    return _FusedMoE.apply(x_sorted, gate_w, up_w, down_w, counts, row_weight, fp8)
 
 
 def torch_fused_ffn(x_sorted, counts, gate_w, up_w, down_w, row_weight):

@@ -1,0 +1,167 @@
+"""GPU parity of the FP8 (E4M3) MFMA gate/up GEMM.
+
+The reference has no FP8 GEMM (its FP8 dispatch dequantises before the experts, ep_communications.py:100), so the
+kernel is pinned in two steps: (1) tightly against the same arithmetic restated on the CPU -- the oracle's decode
+table gives the exact value of every code, the products and sums are taken in fp32/fp64 -- and (2) at the FP8
+tolerance (rtol 5e-2, relative L2 < 0.05, the bound of tests/test_fp8_dispatch.py:85) against the oracle's bf16 expert
+FFN on the dequantised rows with unquantised weights, which is what the layer computes without the FP8 GEMM.
+"""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode(codes):
+    return torch.from_numpy(O.e4m3_decode_table())[codes.long()].double()
+
+
+def _mk(E, H, I, counts, seed, scale=0.05):
+    g = torch.Generator().manual_seed(seed)
+    N = int(sum(counts))
+    x = torch.randn(N, H, generator=g).bfloat16()
+    gw = (torch.randn(E, I, H, generator=g) * scale).bfloat16()
+    uw = (torch.randn(E, I, H, generator=g) * scale).bfloat16()
+    return x, torch.tensor(counts, dtype=torch.int64), gw, uw
+
+
+def _run(x, counts, gw, uw, keep=True):
+    from picotron_amd.expert_parallel import megakernel as mk
+    from picotron_amd.expert_parallel.ep_communications import _per_token_quant_fp8
+
+    xq, xs = _per_token_quant_fp8(x.cuda())
+    gq, gs = mk.quantize_expert_weights(gw.cuda())
+    uq, us = mk.quantize_expert_weights(uw.cuda())
+    act, inter13 = mk._gate_up_fp8(xq.view(torch.uint8), xs, counts.cuda(), gq, gs, uq, us, keep)
+    return act, inter13, (xq.view(torch.uint8).cpu(), xs.cpu(), gq.cpu(), gs.cpu(), uq.cpu(), us.cpu())
+
+
+def _restated(codes, counts):
+    """[g | u] in fp64 from the exact code values and scales, expert by expert."""
+    xq, xs, gq, gs, uq, us = codes
+    E, I, H = gq.shape
+    xv = _decode(xq)
+    outs, start = [], 0
+    for e, n in enumerate(counts.tolist()):
+        rows = xv[start : start + n]
+        g = rows @ _decode(gq[e]).T * xs[start : start + n, None].double() * gs[e * I : (e + 1) * I][None, :].double()
+        u = rows @ _decode(uq[e]).T * xs[start : start + n, None].double() * us[e * I : (e + 1) * I][None, :].double()
+        outs.append(torch.cat([g, u], dim=1))
+        start += n
+    return torch.cat(outs, dim=0)
+
+
+@pytest.mark.parametrize("E,H,I,counts", [
+    (4, 256, 128, [5, 0, 130, 17]),          # empty expert, a tail, more than one wave row
+    (3, 512, 384, [300, 256, 1]),            # a full tile + tail, an exact tile, a single row
+    (2, 1024, 256, [129, 640]),
+])
+def test_fp8_gate_up_matches_restated_arithmetic(gpu, E, H, I, counts):
+    x, cnt, gw, uw = _mk(E, H, I, counts, seed=E + H)
+    act, inter13, codes = _run(x, cnt, gw, uw)
+    ref = _restated(codes, cnt)
+    got = inter13.float().cpu().double()
+    # fp32 accumulation of exact products, then one rounding to bf16 (half an ulp: up to 2^-8 relative), plus
+    # accumulation-order noise: within one bf16 ulp everywhere
+    tol = 2.0 ** -7 * ref.abs() + 1e-5 * ref.abs().max()
+    assert torch.all((got - ref).abs() <= tol), ((got - ref).abs().max().item(), ref.abs().max().item())
+    # act = bf16(bf16(silu(g)) * u) from the rounded g, u the kernel wrote
+    g, u = inter13[:, :I].float().cpu(), inter13[:, I:].float().cpu()
+    want = ((g * torch.sigmoid(g)).bfloat16().float() * u).bfloat16().float()
+    d = (act.float().cpu() - want).abs()
+    assert torch.all(d <= 2.0 ** -7 * want.abs() + 1e-6), d.max().item()   # sigmoid via fast exp / rcp: one bf16 ulp
+
+
+def test_fp8_gate_up_against_bf16_ffn_on_dequantised_rows(gpu):
+    """The FP8 tolerance: relative L2 < 0.05 and 5e-2 of the output scale elementwise, against the oracle's bf16 GEMMs."""
+    E, H, I, counts = 4, 512, 256, [200, 31, 0, 400]
+    x, cnt, gw, uw = _mk(E, H, I, counts, seed=7)
+    act, _, codes = _run(x, cnt, gw, uw, keep=False)
+    xdq = O.dequant_fp8(*O.quant_fp8(x), torch.bfloat16)
+    outs, start = [], 0
+    for e, n in enumerate(counts):
+        rows = xdq[start : start + n]
+        outs.append(torch.nn.functional.silu(rows @ gw[e].T) * (rows @ uw[e].T))
+        start += n
+    ref = torch.cat(outs).float()
+    got = act.float().cpu()
+    rel = ((got - ref).norm() / ref.norm()).item()
+    assert rel < 0.05, rel
+    assert (got - ref).abs().max().item() <= 5e-2 * ref.abs().max().item()
+    # the dispatch codes the kernel consumed are the oracle's (bit-exact quantiser)
+    oq, osc = O.quant_fp8(x)
+    assert torch.equal(codes[0], oq) and torch.equal(codes[1], osc)
+
+
+def test_fp8_gate_up_rejects_untiled_shapes(gpu):
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel import megakernel as mk
+
+    assert not mk.fp8_gemm_supported(48, 96) and mk.fp8_gemm_supported(4096, 14336) and mk.fp8_gemm_supported(2048, 1408)
+    xq = torch.zeros(4, 48, dtype=torch.uint8, device="cuda")
+    xs = torch.ones(4, device="cuda")
+    wq = torch.zeros(1, 96, 48, dtype=torch.uint8, device="cuda")
+    ws = torch.ones(96, device="cuda")
+    with pytest.raises(_lib.PicomoeError):
+        mk._gate_up_fp8(xq, xs, torch.tensor([4], device="cuda"), wq, ws, wq, ws, False)
+
+
+def test_layer_with_fp8_gemm(gpu):
+    """MoELayer, FP8 dispatch + FP8 gate/up GEMM, forward and backward: outputs within the FP8 tolerance of the
+    oracle's layer with FP8 dispatch (bf16 GEMMs on dequantised rows); same routing; gradients (bf16 backward
+    kernels through the FP8 forward's intermediates) within the same tolerance of the layer without the FP8 GEMM."""
+    import types
+
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer
+
+    T, H, I, E, k = 384, 256, 128, 4, 2
+    cfg = types.SimpleNamespace(hidden_size=H, intermediate_size=I, num_experts=E, num_experts_per_tok=k,
+                                ep_fp8_dispatch=True, ep_fp8_gemm=True)
+    torch.manual_seed(3)
+    moe = MoELayer(cfg).cuda().bfloat16()
+    with torch.no_grad():
+        for p in moe.parameters():
+            p.copy_(torch.randn_like(p) * 0.05)
+    x = torch.randn(1, T, H, generator=torch.Generator().manual_seed(4)).bfloat16()
+    up = torch.randn(1, T, H, generator=torch.Generator().manual_seed(5)).bfloat16()
+
+    def run(fp8_gemm):
+        moe.ep_fp8_gemm = fp8_gemm
+        moe.zero_grad(set_to_none=True)
+        xin = x.cuda().requires_grad_(True)
+        out = moe(xin)
+        (out.float() * up.cuda().float()).sum().backward()
+        grads = {n: p.grad.float().cpu() for n, p in moe.named_parameters()}
+        return out.detach().float().cpu(), xin.grad.float().cpu(), grads
+
+    out8, dx8, g8 = run(True)
+    out16, dx16, g16 = run(False)
+    w = O.LayerWeights(
+        router_w=moe.gate.weight.detach().cpu(), router_b=None,
+        gate_w=torch.stack([e.gate_proj.weight.detach().cpu() for e in moe.local_experts]),
+        up_w=torch.stack([e.up_proj.weight.detach().cpu() for e in moe.local_experts]),
+        down_w=torch.stack([e.down_proj.weight.detach().cpu() for e in moe.local_experts]),
+    )
+    ref, _ = O.moe_forward(x[0], w, k, fp8_dispatch=True)
+    ref = ref.float()
+    assert ((out16[0] - ref).norm() / ref.norm()).item() < 1e-2            # the bf16 path, for scale
+    assert ((out8[0] - ref).norm() / ref.norm()).item() < 0.05
+    assert (out8[0] - ref).abs().max().item() <= 5e-2 * ref.abs().max().item()
+    assert ((dx8 - dx16).norm() / dx16.norm()).item() < 0.05
+    for name in g16:
+        if g16[name].norm() > 0:
+            assert ((g8[name] - g16[name]).norm() / g16[name].norm()).item() < 0.05, name
+    # eval mode keeps the quantised weights until a parameter changes
+    moe.eval()
+    moe.ep_fp8_gemm = True
+    with torch.no_grad():
+        a = moe(x.cuda())
+        cached = moe._fp8_weights[1][0].data_ptr()
+        b = moe(x.cuda())
+        assert moe._fp8_weights[1][0].data_ptr() == cached and torch.equal(a, b)
+        moe.local_experts[0].gate_proj.weight.mul_(2.0)
+        c = moe(x.cuda())
+        assert not torch.equal(a, c)
