@@ -26,6 +26,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# L2 <-> memory bytes of the grouped-GEMM launches of one layer step, from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE x 2 KiB, WRITE_SIZE x 1 KiB; factors from the --traffic-probe copy kernel).  Algorithmic: 15.5e9.
+MEASURED_TRAFFIC_BYTES = {"c5": 36.1e9}
 
 WORKLOADS = {
     # name: tokens, hidden, ffn, experts, top_k, shared, capacity_factor, fp8_dispatch, backward
@@ -372,7 +375,7 @@ def main():
         achieved = total_flop / total_ms / 1e9  # TFLOP/s
         result["roofline"] = {
             "bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": "ffn_mfma_kernel (grouped SwiGLU GEMMs: %s)" % ", ".join(kt),
             "flop_per_step": total_flop, "gemm_ms_per_step": total_ms,
             "launches": {k: {"ms": t, "tflops": f / t / 1e9} for k, (t, f) in kt.items()},
