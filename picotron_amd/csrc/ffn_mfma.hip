@@ -1,8 +1,8 @@
 // bf16 MFMA expert-FFN kernels for gfx950 (MI355X): grouped GEMMs over variable-length expert
 // segments, forward + dgrad + wgrad, with the SwiGLU forward / backward fused into the epilogues.
 //
-// Block tile 256 x 256 x 64 (M x N x K), 4 wavefronts (one per SIMD), each owning a 128 x 128
-// sub-tile as 4 x 4 v_mfma_f32_32x32x16_bf16 accumulators (256 fp32 per lane, in AGPRs).  Operand
+// Block tile 256 x 256 x 64 (M x N x K), 8 wavefronts (two per SIMD), each owning a 128 x 64
+// sub-tile as 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (128 fp32 per lane).  Operand
 // tiles go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of
 // 64 KB; a stage is refilled right after the barrier that frees it, half of the loads there and half
 // one k-sub-step later, interleaved with MFMAs so the in-order wave never blocks on the memory queue.
@@ -107,9 +107,7 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
     tc->a_si = r2 / hm;
     tc->b_sn = hm;
     tc->b_si = r2 % hm;
-    int64_t start = 0;
-    for (int i = 0; i < e; ++i) start += counts[i];
-    tc->row0 = start;
+    tc->row0 = segment_start(counts, e);
     tc->rows = (int)counts[e];
     return true;
 }

@@ -35,14 +35,34 @@ struct TileCoord {
 // of at most 128 rows, which cost about half (the wavefronts owning rows 128..255 skip their MFMAs).  Every XCD
 // gets a contiguous run of the heavy tiles followed by a run of the light ones, so the light tiles fill the last,
 // partly occupied round of blocks instead of a full-cost tile being left over there.
+// Wave-wide helpers for the tile lookup: every lane holds one expert's numbers.
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ int wave_scan_i32(int v, int lane) {  // inclusive prefix sum over the 64 lanes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int o = __shfl_up(v, off, 64);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+// The lookup runs once per block in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[]
+// per pass instead of a chain of dependent scalar loads.  Tile and row totals fit 32 bits (the grid does).
 __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, TileCoord* tc) {
-    int64_t heavy_m = 0, light_m = 0;
-    for (int e = 0; e < E; ++e) {
-        const int64_t c = counts[e], rem = c % BM;
+    const int lane = threadIdx.x & 63;
+    int heavy_m = 0, light_m = 0;
+    for (int base = 0; base < E; base += 64) {
+        const int c = base + lane < E ? (int)counts[base + lane] : 0, rem = c % BM;
         heavy_m += c / BM + (rem > BM / 2);
         light_m += (rem > 0 && rem <= BM / 2);
     }
-    const int64_t heavy = heavy_m * n_tiles, light = light_m * n_tiles;
+    heavy_m = wave_sum_i32(heavy_m);
+    light_m = wave_sum_i32(light_m);
+    const int64_t heavy = (int64_t)heavy_m * n_tiles, light = (int64_t)light_m * n_tiles;
     const int64_t heavy_per_xcd = (heavy + kNumXcd - 1) / kNumXcd, light_per_xcd = (light + kNumXcd - 1) / kNumXcd;
     const int64_t xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     bool want_light;
@@ -58,30 +78,44 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
     } else {
         return false;
     }
-    int64_t start = 0;
-    for (int e = 0; e < E; ++e) {
-        const int64_t c = counts[e], full = c / BM, rem = c % BM;
-        const bool light_tail = rem > 0 && rem <= BM / 2;
-        const int64_t me = want_light ? (int64_t)light_tail : full + (rem > BM / 2);
-        const int64_t te = me * n_tiles;
-        if (L < te) {
-            const int m = want_light ? (int)full : (int)(L % me);
-            tc->e = e;
+    int64_t tiles_before = 0, rows_before = 0;
+    for (int base = 0; base < E; base += 64) {
+        const int c = base + lane < E ? (int)counts[base + lane] : 0, full = c / BM, rem = c % BM;
+        const int me = want_light ? (int)(rem > 0 && rem <= BM / 2) : full + (rem > BM / 2);
+        const int te = me * n_tiles;
+        const int te_incl = wave_scan_i32(te, lane), rows_incl = wave_scan_i32(c, lane);
+        const int te_total = __shfl(te_incl, 63, 64);
+        if (L < tiles_before + te_total) {  // the tile belongs to an expert of this group of 64
+            const uint64_t hit = __ballot(tiles_before + te_incl > L);
+            const int src = __ffsll((unsigned long long)hit) - 1;
+            const int c_e = __shfl(c, src, 64), me_e = __shfl(me, src, 64);
+            const int64_t Le = L - tiles_before - (__shfl(te_incl, src, 64) - __shfl(te, src, 64));
+            const int64_t start = rows_before + (__shfl(rows_incl, src, 64) - c_e);
+            const int m = want_light ? c_e / BM : (int)(Le % me_e);
+            tc->e = base + src;
             tc->m_tile = m;
-            tc->n_tile = (int)(L / me);
+            tc->n_tile = (int)(Le / me_e);
             tc->row0 = start + (int64_t)m * BM;
-            const int64_t left = c - (int64_t)m * BM;
-            tc->rows = left < BM ? (int)left : BM;
+            const int left = c_e - m * BM;
+            tc->rows = left < BM ? left : BM;
             tc->a_sn = n_tiles < 4 ? n_tiles : 4;
             tc->a_si = tc->n_tile % tc->a_sn;
-            tc->b_sn = me < 8 ? (int)me : 8;
+            tc->b_sn = me_e < 8 ? me_e : 8;
             tc->b_si = m % tc->b_sn;
             return true;
         }
-        L -= te;
-        start += c;
+        tiles_before += te_total;
+        rows_before += __shfl(rows_incl, 63, 64);
     }
     return false;
+}
+
+// first row of expert e's segment: the sum of the counts before it
+__device__ __forceinline__ int64_t segment_start(const int64_t* counts, int e) {
+    const int lane = threadIdx.x & 63;
+    int64_t start = 0;
+    for (int base = 0; base < e; base += 64) start += wave_sum_i32(base + lane < e ? (int)counts[base + lane] : 0);
+    return start;
 }
 
 

@@ -123,6 +123,29 @@ def test_bf16_ragged_against_oracle(gpu, H, I, counts):
         assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
 
 
+def test_bf16_many_experts(gpu):
+    """150 experts (more than one wave's worth in the tile lookup), counts 0..300 incl. empty experts, full tiles and
+    tails of both classes: forward and gradients against the oracle."""
+    from picotron_amd.expert_parallel import megakernel
+
+    E, H, I = 150, 256, 128
+    gen = torch.Generator().manual_seed(11)
+    counts = torch.randint(0, 40, (E,), generator=gen).tolist()
+    for e, c in ((3, 0), (64, 300), (65, 256), (66, 129), (149, 257), (100, 0)):
+        counts[e] = c
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.bfloat16, 12, scale=0.05)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw)]
+    y = megakernel.fused_moe(leaves[0], cnt.cuda(), *leaves[1:])
+    yr = O.expert_ffn(x, cnt, gw, uw, dw)
+    assert (y.cpu().float() - yr.float()).abs().max() <= 1e-2 * yr.float().abs().max()
+    dy = torch.randn(y.shape, generator=g).bfloat16()
+    y.backward(dy.cuda())
+    ref = O.expert_ffn_backward(x.float(), cnt, gw.float(), uw.float(), dw.float(), dy.float())
+    for got, want in zip([l.grad for l in leaves], ref):
+        assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
+    assert torch.all(leaves[1].grad[3] == 0) and torch.all(leaves[3].grad[100] == 0)   # empty experts
+
+
 def test_mlp_module_runs_the_kernels(gpu):
     import types
 
