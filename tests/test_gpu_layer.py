@@ -363,3 +363,61 @@ def test_fine_grained_skewed_capacity_full_size(gpu):
     dropped_tokens = torch.nonzero((~keep).view(-1, w["k"]).any(1)).squeeze(1)[:8].tolist()
     _sample_check(moe, x, out, ridx, wts.cpu(), keep, sample + dropped_tokens, rtol=1e-2)
     assert int(ties.sum()) >= 0
+
+
+def test_training_steps_follow_the_oracle(gpu):
+    """Two residual MoE blocks (routed + shared experts, aux loss 0.01) trained for four SGD steps, fp32: the loss of
+    every step and the final parameters follow the same loop run on the CPU through the oracle with torch autograd
+    (how the layer sits in picotron's DecoderLayer, model.py:329-331, and train step, train.py:73), the per-expert
+    parameters keep receiving their gradients through the stacked buffers, and the state dict round-trips."""
+    from picotron_amd.expert_parallel.expert_parallel import collect_aux_loss
+
+    cfg = make_config(hidden=32, inter=64, num_experts=4, top_k=2, n_shared=1, router_aux_loss_coef=0.01)
+    blocks = torch.nn.ModuleList([build(cfg, seed=s, std=0.15) for s in (1, 2)])
+    blocks.train()
+    ws = [oracle_weights(b) for b in blocks]
+    for w in ws:
+        for t in w.tensors():
+            t.requires_grad_(True)
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn(2, 48, 32, generator=gen)
+    target = torch.randn(2, 48, 32, generator=gen)
+    lr = 0.02
+    opt = torch.optim.SGD(blocks.parameters(), lr=lr)
+    losses = []
+    for step in range(4):
+        # device
+        opt.zero_grad(set_to_none=True)
+        h = x.cuda()
+        for b in blocks:
+            h = h + b(h)
+        loss = (h - target.cuda()).pow(2).mean() + collect_aux_loss(blocks)
+        loss.backward()
+        opt.step()
+        # oracle
+        ho = x.view(-1, 32)
+        aux = 0.0
+        for w in ws:
+            out, info = O.moe_forward(ho, w, 2, aux_coef=0.01, training=True)
+            ho = ho + out
+            aux = aux + info["aux"]
+        loss_o = (ho - target.view(-1, 32)).pow(2).mean() + aux
+        grads = torch.autograd.grad(loss_o, [t for w in ws for t in w.tensors()])
+        with torch.no_grad():
+            for t, g in zip([t for w in ws for t in w.tensors()], grads):
+                t -= lr * g
+        assert abs(loss.item() - loss_o.item()) <= 2e-5 * abs(loss_o.item()), (step, loss.item(), loss_o.item())
+        losses.append(loss.item())
+    assert losses[-1] < losses[0] - 0.1                                              # and it trains
+    for b, w in zip(blocks, ws):
+        got = oracle_weights(b)
+        for a, r in zip(got.tensors(), w.tensors()):
+            assert (a - r.detach()).abs().max().item() <= 1e-4 * r.detach().abs().max().item() + 1e-6
+    # every per-expert parameter moved (its .grad came through the stacked buffer) and the state dict round-trips
+    sd = blocks[0].state_dict()
+    assert {"gate.weight", "local_experts.3.down_proj.weight", "shared_expert.up_proj.weight", "expert_bias"} <= set(sd)
+    fresh = build(cfg, seed=5, std=0.15)
+    fresh.load_state_dict(sd)
+    fresh.eval(); blocks[0].eval()
+    with torch.no_grad():
+        assert torch.equal(fresh(x.cuda()), blocks[0](x.cuda()))
