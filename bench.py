@@ -5,7 +5,7 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input.  The default workload is the
 Mixtral-shape MoE layer forward + backward with FP8 dispatch (8192 tokens, hidden 4096, FFN 14336, 8 experts,
-top-2, bf16, aux-loss coefficient 0.01): zero_grad, forward, loss = <out, g> + aux, backward -- every gradient
+top-2, bf16, aux-loss coefficient 0.01): zero_grad, forward, backward of loss = <out, g> + aux -- every gradient
 the reference's autograd produces (input, router, 3 x 8 expert matrices) is computed inside the timed region.
 Inputs and weights are resident in HBM before the clock starts.
 
@@ -311,11 +311,13 @@ def main():
             moe.zero_grad(set_to_none=True)
             x.grad = None
             out = moe(x)
-            loss = (out.float() * upstream.float()).sum()
             aux = collect_aux_loss(moe)
+            # backward of loss = <out, g> + aux: d loss / d out = g, d loss / d aux = 1 (the inner product itself is not
+            # part of the layer and is not formed)
             if aux is not None:
-                loss = loss + aux
-            loss.backward()
+                torch.autograd.backward([out, aux], [upstream, torch.ones_like(aux)])
+            else:
+                out.backward(upstream)
         else:
             with torch.no_grad():
                 moe(x)

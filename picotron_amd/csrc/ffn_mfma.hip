@@ -414,7 +414,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     _Pragma("unroll") for (int s_ = 0; s_ < kGroups; ++s_) {                      \
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        \
         __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerGroup, 0);           \
-        if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
+        if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, WITH_LOADS, 0); \
     }                                                                             \
     __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kGroups, 0);
 
@@ -445,18 +445,18 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         if (tail) mask_tail(kt, 0, 0);
         read_frags(1, 1, active);
         mma(0, active);
-        PICOMOE_INTERLEAVE(true)
+        PICOMOE_INTERLEAVE(1)
         __builtin_amdgcn_sched_barrier(0);
         prefetch_l2(kt);
         if (tail) mask_tail(kt, 1, 1);
         read_frags(2, 0, active);
         mma(1, active);
-        PICOMOE_INTERLEAVE(kPrefetchDist > 0)
+        PICOMOE_INTERLEAVE(kPrefetchDist > 0 ? 1 : 0)
         __builtin_amdgcn_sched_barrier(0);
         if (tail) mask_tail(kt, 2, 0);
         read_frags(3, 1, active);
         mma(0, active);
-        PICOMOE_INTERLEAVE(false)
+        PICOMOE_INTERLEAVE(0)
         __builtin_amdgcn_sched_barrier(0);
         // Every wave holds its last fragments of this stage in registers and the next tile has landed:
         // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         flip_stage();
         read_frags(0, 0, active);  // past the last tile this reads a stage that is not used any more
         mma(1, active);
-        PICOMOE_INTERLEAVE(true)
+        PICOMOE_INTERLEAVE(1)
         __builtin_amdgcn_sched_barrier(0);
     }
     };

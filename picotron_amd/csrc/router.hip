@@ -16,6 +16,7 @@ namespace {
 
 constexpr int kMaxTopK = 16;
 constexpr int kRouteBlock = 256;
+constexpr int kMaxExperts = 1024;  // the entry points refuse more
 
 template <typename T>
 __device__ __forceinline__ float to_f32(T v);
@@ -139,9 +140,16 @@ __global__ __launch_bounds__(kRouteBlock) void route_fwd_kernel(const T* __restr
     }
 
     if (counts) {
+        // per-block histogram in LDS first: one global atomic per expert and block instead of one per thread
+        __shared__ int blk_counts[kMaxExperts];
+        for (int e = threadIdx.x; e < E; e += kRouteBlock) blk_counts[e] = 0;
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < EPL; ++i)
-            if (picked[i] && gl + G * i < E) atomicAdd(counts + gl + G * i, picked[i]);
+            if (picked[i] && gl + G * i < E) atomicAdd(blk_counts + gl + G * i, picked[i]);
+        __syncthreads();
+        for (int e = threadIdx.x; e < E; e += kRouteBlock)
+            if (blk_counts[e]) atomicAdd(counts + e, blk_counts[e]);
     }
     if (colsum_partial) {
         __shared__ float acc[kRouteBlock * EPL];
@@ -230,16 +238,29 @@ __global__ __launch_bounds__(256) void balance_kernel(const int* __restrict__ co
                                                       int64_t n_tokens, int E, int k, float aux_coef, float bias_rate,
                                                       float* __restrict__ aux_out, float* __restrict__ bias) {
     __shared__ float red[256];
+    __shared__ float colsum[kMaxExperts];
+    if (aux_out && colsum_partial) {
+        // column sums of the probabilities: each expert's partials are split over kSplit threads (fixed split and a
+        // fixed-order tree, so the result does not depend on timing), 256 / kSplit experts at a time
+        constexpr int kSplit = 32;
+        const int sub = threadIdx.x % kSplit;
+        for (int e0 = 0; e0 < E; e0 += 256 / kSplit) {
+            const int e = e0 + threadIdx.x / kSplit;
+            float cs = 0.f;
+            if (e < E)
+                for (int b = sub; b < n_partials; b += kSplit) cs += colsum_partial[(int64_t)b * E + e];
+#pragma unroll
+            for (int off = kSplit / 2; off > 0; off >>= 1) cs += __shfl_xor(cs, off, kWave);
+            if (e < E && sub == 0) colsum[e] = cs;
+        }
+        __syncthreads();
+    }
     float local_fp = 0.f, local_load = 0.f;
     const float f_scale = (float)((double)E / ((double)k * (double)n_tokens));
     for (int e = threadIdx.x; e < E; e += 256) {
         const float load = (float)counts[e];
         local_load += load;
-        if (aux_out && colsum_partial) {
-            float cs = 0.f;
-            for (int b = 0; b < n_partials; ++b) cs += colsum_partial[(int64_t)b * E + e];
-            local_fp += (load * f_scale) * (cs / (float)n_tokens);
-        }
+        if (aux_out && colsum_partial) local_fp += (load * f_scale) * (colsum[e] / (float)n_tokens);
     }
     red[threadIdx.x] = local_fp;
     __syncthreads();
