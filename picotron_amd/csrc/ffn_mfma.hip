@@ -32,6 +32,11 @@ constexpr int BK = 64;
 #define PICOMOE_MFMA_WAVES 8
 #endif
 constexpr int kWaves = PICOMOE_MFMA_WAVES;
+// modes (bit mask) whose k-loop runs the ping-pong schedule: measured faster for the two dgrad kernels (their B
+// fragments come from transpose reads, twice the LDS instructions per fragment), the same or slower elsewhere
+#ifndef PICOMOE_PINGPONG_MODES
+#define PICOMOE_PINGPONG_MODES ((1 << 2) | (1 << 3))
+#endif
 #ifndef PICOMOE_PREFETCH_FWD
 #define PICOMOE_PREFETCH_FWD 0
 #endif
@@ -117,6 +122,7 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
+    constexpr bool kPingPong = NW == 8 && ((PICOMOE_PINGPONG_MODES >> MODE) & 1);
     constexpr int NI = 4;               // 32-row blocks per wave
     constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
     constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
@@ -431,7 +437,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        if (wave_active) read_frags(0, 0, std::true_type{});
+        if (!kPingPong && wave_active) read_frags(0, 0, std::true_type{});
     }
     auto k_loop = [&](auto active) {
     for (int kt = 0; kt < n_kt; ++kt) {
@@ -473,10 +479,55 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         __builtin_amdgcn_sched_barrier(0);
     }
     };
+    // Ping-pong variant of the loop.  The eight waves form two groups, one wave of every SIMD in each (waves 0-3 own tile
+    // rows 0..127, waves 4-7 rows 128..255).  A k-sub-step is split into a memory phase (the fragment reads of the
+    // sub-step, some of the operand loads of the next k-tile) and an MFMA phase (its 8 MFMAs back to back), every phase
+    // ends in a barrier, and the second group runs one phase behind the first: while one wave of a SIMD issues MFMAs
+    // the other one reads LDS, and the MFMA pipe goes from one group's 8 MFMAs straight to the other's.  (With both
+    // waves running the same finely interleaved stream the older wave of a SIMD wins every MFMA slot, reaches the
+    // per-k-step barrier early and idles there a third of the time while the younger one finishes alone.)
+    auto k_loop_pp = [&](auto active) {
+        auto phase_end = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if (wm == 1) phase_end();  // the phase offset of the second group
+        for (int kt = 0; kt < n_kt; ++kt) {
+            const int stage = kt & 1;
+            const bool tail = MODE == kWgrad && kt == n_kt - 1;
+            const int kt_next = kt + 1 < n_kt ? kt + 1 : n_kt - 1;  // its stage was last read one k-step ago
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                // memory phase
+                read_frags(kk, 0, active);
+                if (kk < 2) issue_loads_part(kt_next, stage ^ 1, kk, active);
+                if (kk == 2) prefetch_l2(kt);
+                if (kk == 3) {
+                    // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
+                    if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+                    else __builtin_amdgcn_s_waitcnt(0x0F71);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (tail) mask_tail(kt, kk, 0);
+                phase_end();
+                // MFMA phase
+                mma(0, active);
+                if (kk == 3) flip_stage();
+                phase_end();
+            }
+        }
+        if (wm == 0) phase_end();  // the first group finishes one phase early
+    };
     // Two copies of the loop, picked per wave: waves that own rows of the tile run all of it; a wave whose 128 rows lie
     // past the end of a short tail only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).
-    if (wave_active) k_loop(std::true_type{});
-    else k_loop(std::false_type{});
+    if (kPingPong) {
+        if (wave_active) k_loop_pp(std::true_type{});
+        else k_loop_pp(std::false_type{});
+    } else {
+        if (wave_active) k_loop(std::true_type{});
+        else k_loop(std::false_type{});
+    }
 #undef PICOMOE_INTERLEAVE
     // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
     __builtin_amdgcn_s_waitcnt(0x0F70);
