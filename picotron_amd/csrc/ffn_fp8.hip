@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
     constexpr int NI = 4, NJ = 2, kWaveCols = 4, CW = 64, QN = 4, RPW = 32;
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
-    if (!locate_m_grouped(p.counts, p.E, p.n_tiles, &tc)) return;
+    if (!locate_m_grouped(p.counts, p.E, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -83,9 +83,8 @@ __device__ __forceinline__ s16x4_t lds_read_tr(const char* p) {
 }
 
 // Logical tile id of this block with the XCD remap, or -1.
-__device__ __forceinline__ int64_t logical_tile(int64_t total) {
+__device__ __forceinline__ int64_t logical_tile(int64_t total, int64_t slot) {
     const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
-    const int64_t slot = blockIdx.x / kNumXcd;
     if (slot >= per_xcd) return -1;
     const int64_t L = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
     return L < total ? L : -1;
@@ -94,9 +93,9 @@ __device__ __forceinline__ int64_t logical_tile(int64_t total) {
 // wgrad tiles: expert by expert; inside an expert the P x Q tile grid is walked in bands of 4 tile columns and, inside
 // a band, in groups of 8 tile rows (tile row fastest inside a group), so that any 32 consecutive tiles -- what one
 // XCD's 32 CUs run at a time -- form an 8 x 4 patch that needs only 8 + 4 operand slices per k-step from its L2.
-__device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, TileCoord* tc) {
+__device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, int64_t slot, TileCoord* tc) {
     const int64_t per_e = (int64_t)m_tiles * n_tiles;
-    const int64_t L = logical_tile(per_e * E);
+    const int64_t L = logical_tile(per_e * E, slot);
     if (L < 0) return false;
     const int e = (int)(L / per_e);
     const int rem = (int)(L % per_e);
@@ -113,7 +112,7 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
     tc->b_sn = hm;
     tc->b_si = r2 % hm;
     tc->row0 = segment_start(counts, e);
-    tc->rows = (int)counts[e];
+    tc->rows = uniform_i32((int)counts[e]);
     return true;
 }
 
@@ -133,9 +132,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
     if (MODE == kWgrad) {
-        if (!locate_wgrad(p.counts, p.E, p.m_tiles, p.n_tiles, &tc)) return;
+        if (!locate_wgrad(p.counts, p.E, p.m_tiles, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
     } else {
-        if (!locate_m_grouped(p.counts, p.E, p.n_tiles, &tc)) return;
+        if (!locate_m_grouped(p.counts, p.E, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
     }
 
     const int tid = threadIdx.x, lane = tid & 63;

@@ -22,6 +22,13 @@ __device__ __forceinline__ void load16_to_lds(const void* g, char* l) {
 }
 
 
+__device__ __forceinline__ int uniform_i32(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 struct TileCoord {
     int e, n_tile, m_tile, rows;  // rows: valid M rows (M-grouped) or valid K rows (wgrad)
     int64_t row0;                 // first row of the tile (M-grouped) or of the expert segment (wgrad)
@@ -50,9 +57,10 @@ __device__ __forceinline__ int wave_scan_i32(int v, int lane) {  // inclusive pr
     return v;
 }
 
-// The lookup runs once per block in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[]
-// per pass instead of a chain of dependent scalar loads.  Tile and row totals fit 32 bits (the grid does).
-__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, TileCoord* tc) {
+// The lookup runs in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[] per pass instead
+// of a chain of dependent scalar loads.  Tile and row totals fit 32 bits.  `slot` is the position of the wanted tile
+// in this block's XCD's run of tiles (blockIdx.x / 8).
+__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, int64_t slot, TileCoord* tc) {
     const int lane = threadIdx.x & 63;
     int heavy_m = 0, light_m = 0;
     for (int base = 0; base < E; base += 64) {
@@ -60,11 +68,11 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
         heavy_m += c / BM + (rem > BM / 2);
         light_m += (rem > 0 && rem <= BM / 2);
     }
-    heavy_m = wave_sum_i32(heavy_m);
-    light_m = wave_sum_i32(light_m);
+    heavy_m = uniform_i32(wave_sum_i32(heavy_m));  // the same in every lane: scalar from here on
+    light_m = uniform_i32(wave_sum_i32(light_m));
     const int64_t heavy = (int64_t)heavy_m * n_tiles, light = (int64_t)light_m * n_tiles;
     const int64_t heavy_per_xcd = (heavy + kNumXcd - 1) / kNumXcd, light_per_xcd = (light + kNumXcd - 1) / kNumXcd;
-    const int64_t xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int64_t xcd = blockIdx.x % kNumXcd;
     bool want_light;
     int64_t L;
     if (slot < heavy_per_xcd) {
@@ -84,28 +92,29 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
         const int me = want_light ? (int)(rem > 0 && rem <= BM / 2) : full + (rem > BM / 2);
         const int te = me * n_tiles;
         const int te_incl = wave_scan_i32(te, lane), rows_incl = wave_scan_i32(c, lane);
-        const int te_total = __shfl(te_incl, 63, 64);
+        const int te_total = uniform_i32(__shfl(te_incl, 63, 64));
         if (L < tiles_before + te_total) {  // the tile belongs to an expert of this group of 64
             const uint64_t hit = __ballot(tiles_before + te_incl > L);
-            const int src = __ffsll((unsigned long long)hit) - 1;
+            const int src = uniform_i32(__ffsll((unsigned long long)hit) - 1);
             const int c_e = __shfl(c, src, 64), me_e = __shfl(me, src, 64);
             const int64_t Le = L - tiles_before - (__shfl(te_incl, src, 64) - __shfl(te, src, 64));
             const int64_t start = rows_before + (__shfl(rows_incl, src, 64) - c_e);
             const int m = want_light ? c_e / BM : (int)(Le % me_e);
-            tc->e = base + src;
-            tc->m_tile = m;
-            tc->n_tile = (int)(Le / me_e);
-            tc->row0 = start + (int64_t)m * BM;
+            // every lane holds the same numbers: hand them out as wave-uniform (scalar) values
+            tc->e = uniform_i32(base + src);
+            tc->m_tile = uniform_i32(m);
+            tc->n_tile = uniform_i32((int)(Le / me_e));
+            tc->row0 = uniform_i64(start + (int64_t)m * BM);
             const int left = c_e - m * BM;
-            tc->rows = left < BM ? left : BM;
+            tc->rows = uniform_i32(left < BM ? left : BM);
             tc->a_sn = n_tiles < 4 ? n_tiles : 4;
             tc->a_si = tc->n_tile % tc->a_sn;
-            tc->b_sn = me_e < 8 ? me_e : 8;
-            tc->b_si = m % tc->b_sn;
+            tc->b_sn = uniform_i32(me_e < 8 ? me_e : 8);
+            tc->b_si = tc->m_tile % tc->b_sn;
             return true;
         }
         tiles_before += te_total;
-        rows_before += __shfl(rows_incl, 63, 64);
+        rows_before += uniform_i32(__shfl(rows_incl, 63, 64));
     }
     return false;
 }
@@ -115,7 +124,7 @@ __device__ __forceinline__ int64_t segment_start(const int64_t* counts, int e) {
     const int lane = threadIdx.x & 63;
     int64_t start = 0;
     for (int base = 0; base < e; base += 64) start += wave_sum_i32(base + lane < e ? (int)counts[base + lane] : 0);
-    return start;
+    return uniform_i64(start);
 }
 
 
