@@ -34,8 +34,12 @@ constexpr int BK = 64;
 constexpr int kWaves = PICOMOE_MFMA_WAVES;
 // modes (bit mask) whose k-loop runs the ping-pong schedule: measured faster for the two dgrad kernels (their B
 // fragments come from transpose reads, twice the LDS instructions per fragment), the same or slower elsewhere
-#ifndef PICOMOE_PINGPONG_MODES
-#define PICOMOE_PINGPONG_MODES ((1 << 2) | (1 << 3))
+// k-loop schedule per mode (two bits each, mode 0 in the low bits): 0 = interleaved, 1 = ping-pong with one k-sub-step
+// per phase, 2 = ping-pong with two.  Measured side by side in one run: the interleaved loop wins for the two forward
+// kernels (K-major operands, one LDS read per fragment), the narrow ping-pong for the two dgrad kernels, the wide one
+// for wgrad (both operands through transpose reads: twelve LDS reads per sub-step).
+#ifndef PICOMOE_LOOP_SCHEDULES
+#define PICOMOE_LOOP_SCHEDULES ((0 << 0) | (0 << 2) | (1 << 4) | (1 << 6) | (2 << 8))
 #endif
 #ifndef PICOMOE_PREFETCH_FWD
 #define PICOMOE_PREFETCH_FWD 0
@@ -121,7 +125,9 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
-    constexpr bool kPingPong = NW == 8 && ((PICOMOE_PINGPONG_MODES >> MODE) & 1);
+    constexpr int kSchedule = NW == 8 ? ((PICOMOE_LOOP_SCHEDULES >> (2 * MODE)) & 3) : 0;
+    constexpr bool kPingPong = kSchedule != 0;
+    constexpr bool kWidePhases = kSchedule == 2;
     constexpr int NI = 4;               // 32-row blocks per wave
     constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
     constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
@@ -496,24 +502,49 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             const int stage = kt & 1;
             const bool tail = MODE == kWgrad && kt == n_kt - 1;
             const int kt_next = kt + 1 < n_kt ? kt + 1 : n_kt - 1;  // its stage was last read one k-step ago
+            if constexpr (kWidePhases) {
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                // memory phase
-                read_frags(kk, 0, active);
-                if (kk < 2) issue_loads_part(kt_next, stage ^ 1, kk, active);
-                if (kk == 2) prefetch_l2(kt);
-                if (kk == 3) {
-                    // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
-                    if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-                    else __builtin_amdgcn_s_waitcnt(0x0F71);
+                for (int half = 0; half < 2; ++half) {
+                    // memory phase: the fragments of two sub-steps
+                    read_frags(2 * half, 0, active);
+                    read_frags(2 * half + 1, 1, active);
+                    if (half == 0) {
+                        issue_loads_part(kt_next, stage ^ 1, 0, active);
+                        issue_loads_part(kt_next, stage ^ 1, 1, active);
+                    } else {
+                        prefetch_l2(kt);
+                        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+                        else __builtin_amdgcn_s_waitcnt(0x0F71);
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (tail) { mask_tail(kt, 2 * half, 0); mask_tail(kt, 2 * half + 1, 1); }
+                    phase_end();
+                    // MFMA phase: 16 MFMAs
+                    mma(0, active);
+                    mma(1, active);
+                    if (half == 1) flip_stage();
+                    phase_end();
                 }
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (tail) mask_tail(kt, kk, 0);
-                phase_end();
-                // MFMA phase
-                mma(0, active);
-                if (kk == 3) flip_stage();
-                phase_end();
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    // memory phase
+                    read_frags(kk, 0, active);
+                    if (kk < 2) issue_loads_part(kt_next, stage ^ 1, kk, active);
+                    if (kk == 2) prefetch_l2(kt);
+                    if (kk == 3) {
+                        // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
+                        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+                        else __builtin_amdgcn_s_waitcnt(0x0F71);
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (tail) mask_tail(kt, kk, 0);
+                    phase_end();
+                    // MFMA phase
+                    mma(0, active);
+                    if (kk == 3) flip_stage();
+                    phase_end();
+                }
             }
         }
         if (wm == 0) phase_end();  // the first group finishes one phase early
