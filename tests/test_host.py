@@ -78,6 +78,38 @@ def test_module_structure_and_defaults():
     assert w.abs().max() <= (1.0 / 32) ** 0.5
 
 
+def test_parameter_names_fit_the_reference_model_code():
+    """The layer sits under ``DecoderLayer.mlp`` (model.py:306); the reference's parameter counting keys on the
+    substrings ``mlp.local_experts.`` / ``mlp.gate.`` / ``mlp.shared_expert.`` (utils.py:82-86) and its checkpoint
+    loader fills parameters missing from a dense checkpoint with zeros and then calls ``reset_parameters()``
+    (checkpoint.py:132-141)."""
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer
+    from picotron_amd.model import MLP
+
+    class Block(torch.nn.Module):
+        def __init__(self, cfg):
+            super().__init__()
+            self.mlp = MoELayer(cfg) if getattr(cfg, "num_experts", 1) > 1 else MLP(cfg)
+
+    block = Block(_cfg(num_shared_experts=1))
+    names = [n for n, _ in block.named_parameters()]
+    experts = [n for n in names if "mlp.local_experts." in n]
+    router = [n for n in names if "mlp.gate." in n]
+    shared = [n for n in names if "mlp.shared_expert." in n]
+    assert len(experts) == 4 * 3 and router == ["mlp.gate.weight"] and len(shared) == 3
+    assert sorted(experts + router + shared) == sorted(names)
+    assert "mlp.local_experts.2.up_proj.weight" in names and "mlp.expert_bias" in block.state_dict()
+    # the zero-fill path: zeros in, proper init out
+    sd = {n: torch.zeros(p.shape) for n, p in block.named_parameters()}
+    sd["mlp.expert_bias"] = torch.zeros(4)
+    block.load_state_dict(sd)
+    assert all(float(p.abs().sum()) == 0.0 for p in block.parameters())
+    block.mlp.reset_parameters()
+    assert all(float(p.abs().sum()) > 0.0 for p in block.parameters())
+    dense = Block(types.SimpleNamespace(hidden_size=16, intermediate_size=32))
+    assert sorted(n for n, _ in dense.named_parameters()) == ["mlp.down_proj.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight"]
+
+
 def test_cpu_tensors_are_refused_not_silently_computed():
     from picotron_amd.expert_parallel import megakernel
     from picotron_amd.expert_parallel.expert_parallel import MoELayer
