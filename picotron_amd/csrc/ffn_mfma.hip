@@ -4,8 +4,8 @@
 // Block tile 256 x 256 x 64 (M x N x K), 8 wavefronts (two per SIMD), each owning a 128 x 64
 // sub-tile as 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (128 fp32 per lane).  Operand
 // tiles go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of
-// 64 KB; a stage is refilled right after the barrier that frees it, half of the loads there and half
-// one k-sub-step later, interleaved with MFMAs so the in-order wave never blocks on the memory queue.
+// 64 KB.  The k-loop is a ping-pong: the two waves of a SIMD alternate between a memory phase (fragment
+// reads, operand loads of the next k-tile, L2 prefetch) and an MFMA phase, one phase apart.
 //
 // Two LDS tile layouts, chosen per operand by how it lies in memory:
 //   K-major  (rows of the operand are contiguous along K: activations, forward weights)
@@ -34,18 +34,17 @@ constexpr int BK = 64;
 constexpr int kWaves = PICOMOE_MFMA_WAVES;
 // modes (bit mask) whose k-loop runs the ping-pong schedule: measured faster for the two dgrad kernels (their B
 // fragments come from transpose reads, twice the LDS instructions per fragment), the same or slower elsewhere
-// k-loop schedule per mode (two bits each, mode 0 in the low bits): 0 = interleaved, 1 = ping-pong with one k-sub-step
-// per phase, 2 = ping-pong with two.  Measured side by side in one run: the interleaved loop wins for the two forward
-// kernels (K-major operands, one LDS read per fragment), the narrow ping-pong for the two dgrad kernels, the wide one
-// for wgrad (both operands through transpose reads: twelve LDS reads per sub-step).
-#ifndef PICOMOE_LOOP_SCHEDULES
-#define PICOMOE_LOOP_SCHEDULES ((0 << 0) | (0 << 2) | (1 << 4) | (1 << 6) | (2 << 8))
+// Modes (bit mask) whose ping-pong k-loop runs two k-sub-steps per phase instead of one.  Measured side by side in one
+// run: one sub-step per phase wins for the forward and dgrad kernels, two for wgrad (both operands come through
+// transpose reads, twelve LDS reads per sub-step).
+#ifndef PICOMOE_WIDE_PHASE_MODES
+#define PICOMOE_WIDE_PHASE_MODES (1 << 4)
 #endif
 #ifndef PICOMOE_PREFETCH_FWD
-#define PICOMOE_PREFETCH_FWD 0
+#define PICOMOE_PREFETCH_FWD 2
 #endif
 #ifndef PICOMOE_PREFETCH_BWD
-#define PICOMOE_PREFETCH_BWD 4
+#define PICOMOE_PREFETCH_BWD 2
 #endif
 
 enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
@@ -125,9 +124,7 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
-    constexpr int kSchedule = NW == 8 ? ((PICOMOE_LOOP_SCHEDULES >> (2 * MODE)) & 3) : 0;
-    constexpr bool kPingPong = kSchedule != 0;
-    constexpr bool kWidePhases = kSchedule == 2;
+    constexpr bool kWidePhases = (PICOMOE_WIDE_PHASE_MODES >> MODE) & 1;
     constexpr int NI = 4;               // 32-row blocks per wave
     constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
     constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
@@ -411,24 +408,6 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
     };
 
-    // One k-sub-step = the fragment reads of the NEXT sub-step (and, in two of the four sub-steps, half of the
-    // direct-to-LDS loads of a later tile) interleaved with the 16 MFMAs of this sub-step.
-    // Scheduling of one k-sub-step: the LDS reads of the NEXT sub-step (and any direct-to-LDS loads) go into
-    // the first half, one after each MFMA (the sub-step starts with an MFMA: the compiler waits for ALL LDS
-    // reads before a sub-step's first MFMA, so no read may sit right in front of it), and the second half
-    // (8 MFMAs, 256 cycles) covers their latency.
-    constexpr int kReads = NI * (T::kAKMajor ? 1 : 2) + NJ * (T::kBKMajor ? 1 : 2);  // LDS reads per sub-step
-    constexpr int kMfmas = NI * NJ;
-    constexpr int kGroups = kMfmas / 2;                                               // MFMAs that get company
-    constexpr int kReadsPerGroup = (kReads + kGroups - 1) / kGroups;
-#define PICOMOE_INTERLEAVE(WITH_LOADS)                                            \
-    _Pragma("unroll") for (int s_ = 0; s_ < kGroups; ++s_) {                      \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        \
-        __builtin_amdgcn_sched_group_barrier(0x100, kReadsPerGroup, 0);           \
-        if (WITH_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, WITH_LOADS, 0); \
-    }                                                                             \
-    __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kGroups, 0);
-
     if (n_kt > 0) {
         issue_loads_part(0, 0, 0, std::false_type{});
         issue_loads_part(0, 0, 1, std::false_type{});
@@ -442,55 +421,15 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        if (!kPingPong && wave_active) read_frags(0, 0, std::true_type{});
     }
-    auto k_loop = [&](auto active) {
-    for (int kt = 0; kt < n_kt; ++kt) {
-        const int stage = kt & 1;
-        const bool tail = MODE == kWgrad && kt == n_kt - 1;
-        __builtin_amdgcn_sched_barrier(0);
-        // second half of the refill begun in the previous k-step.  Issued unconditionally (past the end the tile
-        // index is clamped and the data land in a stage nobody reads) so that the loads sit in the same basic
-        // block as the MFMAs and can be interleaved with them.
-        issue_loads_part(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, 1, active);
-        if (tail) mask_tail(kt, 0, 0);
-        read_frags(1, 1, active);
-        mma(0, active);
-        PICOMOE_INTERLEAVE(1)
-        __builtin_amdgcn_sched_barrier(0);
-        prefetch_l2(kt);
-        if (tail) mask_tail(kt, 1, 1);
-        read_frags(2, 0, active);
-        mma(1, active);
-        PICOMOE_INTERLEAVE(kPrefetchDist > 0 ? 1 : 0)
-        __builtin_amdgcn_sched_barrier(0);
-        if (tail) mask_tail(kt, 2, 0);
-        read_frags(3, 1, active);
-        mma(0, active);
-        PICOMOE_INTERLEAVE(0)
-        __builtin_amdgcn_sched_barrier(0);
-        // Every wave holds its last fragments of this stage in registers and the next tile has landed:
-        // the stage can be refilled (tile kt+2) a full k-step before that tile is needed.
-        // all operand loads have landed; this k-step's prefetch load, the youngest in the queue, may stay in flight
-        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-        else __builtin_amdgcn_s_waitcnt(0x0F71);
-        __syncthreads();
-        issue_loads_part(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0, active);
-        if (tail) mask_tail(kt, 3, 1);
-        flip_stage();
-        read_frags(0, 0, active);  // past the last tile this reads a stage that is not used any more
-        mma(1, active);
-        PICOMOE_INTERLEAVE(1)
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    };
-    // Ping-pong variant of the loop.  The eight waves form two groups, one wave of every SIMD in each (waves 0-3 own tile
+    // The k-loop, a ping-pong between two groups of waves.  The eight waves form two groups, one wave of every SIMD in each (waves 0-3 own tile
     // rows 0..127, waves 4-7 rows 128..255).  A k-sub-step is split into a memory phase (the fragment reads of the
     // sub-step, some of the operand loads of the next k-tile) and an MFMA phase (its 8 MFMAs back to back), every phase
     // ends in a barrier, and the second group runs one phase behind the first: while one wave of a SIMD issues MFMAs
     // the other one reads LDS, and the MFMA pipe goes from one group's 8 MFMAs straight to the other's.  (With both
-    // waves running the same finely interleaved stream the older wave of a SIMD wins every MFMA slot, reaches the
-    // per-k-step barrier early and idles there a third of the time while the younger one finishes alone.)
+    // waves running the same stream, LDS reads and loads interleaved between the MFMAs, the older wave of a SIMD wins
+    // every MFMA slot, reaches the per-k-step barrier early and idles there a third of the time while the younger one
+    // finishes alone: measured with in-kernel cycle counters.)
     auto k_loop_pp = [&](auto active) {
         auto phase_end = [&]() {
             __builtin_amdgcn_sched_barrier(0);
@@ -551,14 +490,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     };
     // Two copies of the loop, picked per wave: waves that own rows of the tile run all of it; a wave whose 128 rows lie
     // past the end of a short tail only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).
-    if (kPingPong) {
-        if (wave_active) k_loop_pp(std::true_type{});
-        else k_loop_pp(std::false_type{});
-    } else {
-        if (wave_active) k_loop(std::true_type{});
-        else k_loop(std::false_type{});
-    }
-#undef PICOMOE_INTERLEAVE
+    if (wave_active) k_loop_pp(std::true_type{});
+    else k_loop_pp(std::false_type{});
     // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
