@@ -1,13 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the single-GPU MoE hot path on MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c4|train_step]
 
 A "step" is one pass of the hot path over one batch of synthetic input.  The default workload is the
 Mixtral-shape MoE layer forward + backward with FP8 dispatch (8192 tokens, hidden 4096, FFN 14336, 8 experts,
 top-2, bf16, aux-loss coefficient 0.01): zero_grad, forward, backward of loss = <out, g> + aux -- every gradient
 the reference's autograd produces (input, router, 3 x 8 expert matrices) is computed inside the timed region.
 Inputs and weights are resident in HBM before the clock starts.
+
+`--workload train_step` instead times a whole optimizer step (forward, cross entropy + aux, backward, AdamW) of a
+4-layer Llama whose feed-forward blocks are this MoE layer, the set-up of the reference's tests/bench_ep_train_step.py.
 
 Prints ONE JSON line on stdout: the layer's tokens/s as `value`, a `roofline` object for the grouped-GEMM
 kernels (algorithmic FLOP / launch durations measured here with events on the launch stream), the FP8
@@ -278,12 +281,67 @@ def cpu_baseline(w, moe, budget_s=25.0):
     }
 
 
+def train_step_bench(args):
+    """One optimizer step of a small Llama with MoE feed-forward blocks, the recipe and default sizes of the
+    reference's tests/bench_ep_train_step.py:27-44, 54-60, 82-93 (hidden 2048, FFN 2048, 4 layers, 16 heads / 4 kv
+    heads, 8 experts top-2 + 1 shared, sequence 2048, micro-batch 1, vocabulary 32000, bf16, AdamW lr 1e-4)."""
+    import torch
+    import torch.nn.functional as F
+
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel.expert_parallel import collect_aux_loss
+    from picotron_amd.model import Llama
+
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    cfg = types.SimpleNamespace(
+        vocab_size=32000, hidden_size=2048, intermediate_size=2048, num_attention_heads=16, num_key_value_heads=4,
+        num_hidden_layers=4, max_position_embeddings=2048, rms_norm_eps=1e-5, rope_theta=10000.0, num_experts=8,
+        num_experts_per_tok=2, num_shared_experts=1, norm_topk_prob=True)
+    seq, mbs = 2048, 1
+    torch.manual_seed(0)
+    model = Llama(cfg).to(torch.bfloat16).cuda().train()
+    optimizer = torch.optim.AdamW(model.parameters(), lr=1e-4)
+    torch.manual_seed(42)
+    input_ids = torch.randint(0, cfg.vocab_size, (mbs, seq), device="cuda")
+    target_ids = torch.randint(0, cfg.vocab_size, (mbs, seq), device="cuda")
+
+    def step():
+        optimizer.zero_grad(set_to_none=True)
+        logits = model(input_ids)
+        loss = F.cross_entropy(logits.view(-1, logits.size(-1)).float(), target_ids.view(-1))
+        aux = collect_aux_loss(model)
+        if aux is not None:
+            loss = loss + aux.float()
+        loss.backward()
+        optimizer.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    n_params = sum(p.numel() for p in model.parameters())
+    log(f"[bench] train_step: {ms:.3f} ms/step, {mbs * seq / ms * 1e3:,.0f} tokens/s, loss {float(loss.detach()):.3f}")
+    print(json.dumps({
+        "metric": "Llama-MoE train-step tokens/s (fwd + loss + bwd + AdamW, 1 GPU)", "value": mbs * seq / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "4-layer Llama, MoE feed-forward (hidden 2048, FFN 2048, 8 experts top-2 + 1 shared), "
+                               "seq 2048 x mbs 1, vocab 32000, AdamW", "tokens": mbs * seq, "parameters": n_params},
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + ["train_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-times", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -292,6 +350,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU (the EP=1 MoE hot path); run with --gpus 1")
+    if args.workload == "train_step":
+        return train_step_bench(args)
 
     import torch
 

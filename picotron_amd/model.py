@@ -1,14 +1,17 @@
-"""The SwiGLU MLP that expert and shared-expert weights live in.
+"""The SwiGLU MLP that expert and shared-expert weights live in, and the decoder the MoE layer is called from.
 
-Mirrors picotron/model.py:236-258 (class ``MLP``): three bias-free linears ``up_proj``, ``gate_proj``,
-``down_proj`` and ``down(silu(gate(x)) * up(x))``.  The forward runs the grouped SwiGLU kernels with
-a single expert; there is no eager path.
+``MLP`` mirrors picotron/model.py:236-258: three bias-free linears ``up_proj``, ``gate_proj``, ``down_proj`` and
+``down(silu(gate(x)) * up(x))``.  Its forward runs the grouped SwiGLU kernels with a single expert; there is no eager
+path.  ``Llama`` / ``DecoderLayer`` / ``Attention`` / ``LlamaRMSNorm`` / ``Embedding`` / ``FinalProjection`` mirror the
+module tree of picotron/model.py:98-402 on one GPU (no tensor, context or pipeline parallel branches) with the
+reference's parameter names; outside ``mlp`` they are library calls (attention, dense GEMMs, norms).
 """
 
 import math
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 
 class MLP(nn.Module):
@@ -34,3 +37,186 @@ class MLP(nn.Module):
             rows, counts, self.gate_proj.weight.unsqueeze(0), self.up_proj.weight.unsqueeze(0), self.down_proj.weight.unsqueeze(0)
         )
         return y.reshape(*lead, y.shape[-1])
+
+
+def rope_tables(seq_length, head_dim, base=500000.0):
+    """cos / sin tables ``[seq_length, head_dim]`` in fp32 (picotron/model.py:39-52): angle ``m * base^(-2i/d)`` for
+    position m and pair i, the half-width table repeated twice along the last axis (the rotate-half convention)."""
+    assert head_dim % 2 == 0
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    angle = torch.arange(seq_length).float().unsqueeze(1) * inv_freq
+    return torch.cos(angle).repeat(1, 2), torch.sin(angle).repeat(1, 2)
+
+
+def apply_rotary_pos_emb(x, cos, sin):
+    """Rotate-half RoPE on ``[B, heads, S, d]`` (picotron/model.py:29-36)."""
+    half = x.shape[-1] // 2
+    rotated = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+    return x * cos + rotated * sin
+
+
+class LlamaRMSNorm(nn.Module):
+    """picotron/model.py:98-116: statistics in fp32, the normalised value cast back before the weight multiplies."""
+
+    def __init__(self, hidden_size, eps=1e-5):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def reset_parameters(self):
+        nn.init.ones_(self.weight)
+
+    def forward(self, hidden_states):
+        h = hidden_states.float()
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * h.to(hidden_states.dtype)
+
+
+def _uniform_fan_in_(weight):
+    bound = math.sqrt(1.0 / weight.size(1))
+    torch.nn.init.uniform_(weight, -bound, bound)
+
+
+class Attention(nn.Module):
+    """Causal grouped-query self-attention, the reference's scaled-dot-product branch (picotron/model.py:118-233 with
+    FLASH_ATTEN=0): bias-free q/k/v/out projections, rotate-half RoPE on q and k, k/v heads repeated to the query
+    heads.  A library attention call: this block is a caller of the MoE layer, not part of it."""
+
+    def __init__(self, config, layer_idx):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_key_values = config.num_key_value_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(self.hidden_size, self.num_key_values * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(self.hidden_size, self.num_key_values * self.head_dim, bias=False)
+        self.out_proj = nn.Linear(self.hidden_size, self.hidden_size, bias=False)
+        self.layer_idx = layer_idx
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        for lin in (self.q_proj, self.k_proj, self.v_proj, self.out_proj):
+            _uniform_fan_in_(lin.weight)
+
+    def forward(self, x, cos, sin, attention_mask=None, position_ids=None):
+        B, S, _ = x.shape
+        heads = lambda t, n: t.view(B, S, n, self.head_dim).transpose(1, 2)
+        q = apply_rotary_pos_emb(heads(self.q_proj(x), self.num_heads), cos, sin)
+        k = apply_rotary_pos_emb(heads(self.k_proj(x), self.num_key_values), cos, sin)
+        v = heads(self.v_proj(x), self.num_key_values)
+        group = self.num_heads // self.num_key_values
+        k, v = k.repeat_interleave(group, dim=1), v.repeat_interleave(group, dim=1)
+        out = F.scaled_dot_product_attention(q, k, v, is_causal=q.size(2) == k.size(2))
+        return self.out_proj(out.transpose(1, 2).reshape(B, S, self.num_heads * self.head_dim))
+
+
+class FinalProjection(nn.Module):
+    """picotron/model.py:261-286: the vocabulary projection as a bare weight ``[vocab, hidden]``."""
+
+    def __init__(self, hidden_size, vocab_size, bias=False):
+        super().__init__()
+        self.in_features, self.out_features = hidden_size, vocab_size
+        self.weight = nn.Parameter(torch.empty(vocab_size, hidden_size))
+        self.bias = nn.Parameter(torch.empty(vocab_size)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        _uniform_fan_in_(self.weight)
+        if self.bias is not None:
+            torch.nn.init.uniform_(self.bias, -math.sqrt(1.0 / self.in_features), math.sqrt(1.0 / self.in_features))
+
+    def forward(self, x):
+        return F.linear(x, self.weight, self.bias)
+
+
+class Embedding(nn.Module):
+    """picotron/model.py:343-360: token embedding table, N(0, 1) init."""
+
+    def __init__(self, num_embeddings, embedding_dim, padding_idx=None):
+        super().__init__()
+        self.num_embeddings, self.embedding_dim, self.padding_idx = num_embeddings, embedding_dim, padding_idx
+        self.weight = nn.Parameter(torch.empty(num_embeddings, embedding_dim))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        torch.nn.init.normal_(self.weight, mean=0.0, std=1.0)
+
+    def forward(self, x):
+        return F.embedding(x, self.weight, self.padding_idx)
+
+
+class DecoderLayer(nn.Module):
+    """picotron/model.py:289-340.  Sequential: norm, attention, residual, norm, mlp, residual.  With
+    ``config.parallel_block`` attention and mlp read one shared norm and both are added to the residual.  ``mlp`` is
+    the MoE layer when ``config.num_experts > 1`` (picotron/model.py:306), the dense SwiGLU MLP otherwise."""
+
+    def __init__(self, config, layer_idx):
+        super().__init__()
+        from picotron_amd.expert_parallel.expert_parallel import MoELayer
+
+        self.parallel_block = getattr(config, "parallel_block", False)
+        self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        if not self.parallel_block:
+            self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.attention = Attention(config, layer_idx=layer_idx)
+        self.mlp = MoELayer(config) if getattr(config, "num_experts", 1) > 1 else MLP(config)
+        self.layer_idx = layer_idx
+        # plain attributes like the reference's (no state_dict entry); cast to the activations' device and dtype on use
+        self.cos, self.sin = rope_tables(
+            config.max_position_embeddings, config.hidden_size // config.num_attention_heads, base=config.rope_theta
+        )
+
+    def _rope(self, x):
+        if self.cos.device != x.device or self.cos.dtype != x.dtype:
+            self.cos, self.sin = self.cos.to(x.device, x.dtype), self.sin.to(x.device, x.dtype)
+        S = x.shape[1]
+        return self.cos[:S], self.sin[:S]
+
+    def forward(self, x, attention_mask=None, position_ids=None):
+        cos, sin = self._rope(x)
+        if self.parallel_block:
+            n = self.input_layernorm(x)
+            return x + self.attention(n, cos, sin, attention_mask, position_ids) + self.mlp(n)
+        x = x + self.attention(self.input_layernorm(x), cos, sin, attention_mask, position_ids)
+        return x + self.mlp(self.post_attention_layernorm(x))
+
+
+class Llama(nn.Module):
+    """picotron/model.py:363-402: embedding, ``decoder_layers``, ``final_norm``, ``final_proj``; same module and
+    parameter names, so a reference state_dict loads unchanged."""
+
+    def __init__(self, config) -> None:
+        super().__init__()
+        assert config.hidden_size % config.num_attention_heads == 0
+        assert config.num_attention_heads % config.num_key_value_heads == 0
+        self.vocab_size = config.vocab_size
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_key_values = config.num_key_value_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        self.max_position_embeddings = config.max_position_embeddings
+        self.num_layers = config.num_hidden_layers
+        self.model_config = config
+        self.embedding = Embedding(self.vocab_size, self.hidden_size)
+        self.decoder_layers = nn.ModuleList([DecoderLayer(config, layer_idx=i) for i in range(self.num_layers)])
+        self.final_proj = FinalProjection(self.hidden_size, self.vocab_size, bias=False)
+        self.final_norm = LlamaRMSNorm(self.hidden_size, eps=config.rms_norm_eps)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.embedding.reset_parameters()
+        for layer in self.decoder_layers:
+            layer.input_layernorm.reset_parameters()
+            layer.attention.reset_parameters()
+            if not layer.parallel_block:
+                layer.post_attention_layernorm.reset_parameters()
+            layer.mlp.reset_parameters()
+        self.final_norm.reset_parameters()
+        self.final_proj.reset_parameters()
+
+    def forward(self, input_ids, attention_mask=None, position_ids=None):
+        x = self.embedding(input_ids)
+        for layer in self.decoder_layers:
+            x = layer(x)
+        return self.final_proj(self.final_norm(x))

@@ -110,6 +110,40 @@ def test_parameter_names_fit_the_reference_model_code():
     assert sorted(n for n, _ in dense.named_parameters()) == ["mlp.down_proj.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight"]
 
 
+def test_llama_module_tree_uses_the_reference_names():
+    """picotron/model.py:363-402: ``embedding``, ``decoder_layers.N.{input_layernorm, post_attention_layernorm,
+    attention.{q,k,v,out}_proj, mlp}``, ``final_proj``, ``final_norm``.  The reference's parameter counting keys on the
+    substrings "attention", "mlp", "embed", "final_proj" (utils.py:88) besides the MoE ones; RoPE tables are plain
+    attributes, not state (model.py:309-311)."""
+    from picotron_amd.expert_parallel.expert_parallel import MoELayer
+    from picotron_amd.model import MLP, Llama
+
+    cfg = types.SimpleNamespace(vocab_size=50, hidden_size=16, intermediate_size=32, num_attention_heads=4,
+                                num_key_value_heads=2, num_hidden_layers=2, max_position_embeddings=8, rms_norm_eps=1e-5,
+                                rope_theta=10000.0, num_experts=4, num_experts_per_tok=2, num_shared_experts=1)
+    model = Llama(cfg)
+    names = [n for n, _ in model.named_parameters()]
+    per_layer = ["input_layernorm.weight", "post_attention_layernorm.weight", "attention.q_proj.weight",
+                 "attention.k_proj.weight", "attention.v_proj.weight", "attention.out_proj.weight", "mlp.gate.weight"]
+    for i in range(2):
+        for n in per_layer:
+            assert f"decoder_layers.{i}.{n}" in names
+        assert isinstance(model.decoder_layers[i].mlp, MoELayer)
+    assert names[0] == "embedding.weight" and names[-2:] == ["final_proj.weight", "final_norm.weight"]
+    assert model.decoder_layers[0].attention.k_proj.weight.shape == (8, 16)      # 2 kv heads x head_dim 4
+    assert model.decoder_layers[0].cos.shape == (8, 4) and not any("cos" in k for k in model.state_dict())
+    counted = [n for n in names if any(k in n.lower() for k in ("attention", "mlp", "embed", "final_proj"))]
+    assert sorted(set(names) - set(counted)) == sorted(
+        # "post_attention_layernorm" contains "attention", so the reference counts it with the split parameters
+        [f"decoder_layers.{i}.input_layernorm.weight" for i in range(2)] + ["final_norm.weight"])
+    cfg.parallel_block, cfg.num_experts = True, 1
+    dense = Llama(cfg)
+    assert isinstance(dense.decoder_layers[0].mlp, MLP) and not hasattr(dense.decoder_layers[0], "post_attention_layernorm")
+    # embedding N(0,1), projections uniform in +-1/sqrt(fan_in) (model.py:147-155, 353-354)
+    assert 0.8 < float(dense.embedding.weight.std()) < 1.2
+    assert float(dense.final_proj.weight.abs().max()) <= 0.25
+
+
 def test_cpu_tensors_are_refused_not_silently_computed():
     from picotron_amd.expert_parallel import megakernel
     from picotron_amd.expert_parallel.expert_parallel import MoELayer
