@@ -5,7 +5,8 @@
 // sub-tile as 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (128 fp32 per lane).  Operand
 // tiles go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of
 // 64 KB.  The k-loop is a ping-pong: the two waves of a SIMD alternate between a memory phase (fragment
-// reads, operand loads of the next k-tile, L2 prefetch) and an MFMA phase, one phase apart.
+// reads) and an MFMA phase (8 MFMAs with the operand loads of the next k-tile and the L2 prefetch issued
+// between them), one phase apart.
 //
 // Two LDS tile layouts, chosen per operand by how it lies in memory:
 //   K-major  (rows of the operand are contiguous along K: activations, forward weights)
@@ -32,14 +33,6 @@ constexpr int BK = 64;
 #define PICOMOE_MFMA_WAVES 8
 #endif
 constexpr int kWaves = PICOMOE_MFMA_WAVES;
-// modes (bit mask) whose k-loop runs the ping-pong schedule: measured faster for the two dgrad kernels (their B
-// fragments come from transpose reads, twice the LDS instructions per fragment), the same or slower elsewhere
-// Modes (bit mask) whose ping-pong k-loop runs two k-sub-steps per phase instead of one.  Measured side by side in one
-// run: one sub-step per phase wins for the forward and dgrad kernels, two for wgrad (both operands come through
-// transpose reads, twelve LDS reads per sub-step).
-#ifndef PICOMOE_WIDE_PHASE_MODES
-#define PICOMOE_WIDE_PHASE_MODES (1 << 4)
-#endif
 #ifndef PICOMOE_PREFETCH_FWD
 #define PICOMOE_PREFETCH_FWD 2
 #endif
@@ -124,7 +117,6 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
-    constexpr bool kWidePhases = (PICOMOE_WIDE_PHASE_MODES >> MODE) & 1;
     constexpr int NI = 4;               // 32-row blocks per wave
     constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
     constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
@@ -285,27 +277,29 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         pf_cur += adv;
     };
 
-    // `active` (a std::bool_constant): false in the loop copy of the waves that only load and synchronise
-    auto issue_loads_n = [&](int kt, int stage, int q0, auto nq, auto /*active*/) {
+    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage
+    auto issue_a = [&](int kt, int stage, int q) {
         char* base = lds + stage * kStageBytes;
         const char* ab = a_base + (int64_t)kt * a_step;
-        const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
-#pragma unroll
-        for (int q = q0; q < q0 + decltype(nq)::value; ++q) {
-            const int dk = k_clamp(kt, q);
-            if (T::kAKMajor)
-                load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
-            else
-                load16_to_lds(ab + (uint32_t)(a_off[q] + dk * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
-            if (T::kBKMajor)
-                load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * RPW + q * 8) * 128);
-            else
-                load16_to_lds(bb + (uint32_t)(b_off[q] + dk * (int)p.ldb * 2), base + kTileBytes + (wave * KPW + q * 2) * 512);
-        }
+        if (T::kAKMajor)
+            load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
+        else
+            load16_to_lds(ab + (uint32_t)(a_off[q] + k_clamp(kt, q) * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
     };
-    // half of a wave's loads for one tile: part 0 or 1
-    auto issue_loads_part = [&](int kt, int stage, int part, auto active) {
-        issue_loads_n(kt, stage, part * (QN / 2), std::integral_constant<int, QN / 2>{}, active);
+    auto issue_b = [&](int kt, int stage, int q) {
+        char* base = lds + stage * kStageBytes + kTileBytes;
+        const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
+        if (T::kBKMajor)
+            load16_to_lds(bb + b_off[q], base + (wave * RPW + q * 8) * 128);
+        else
+            load16_to_lds(bb + (uint32_t)(b_off[q] + k_clamp(kt, q) * (int)p.ldb * 2), base + (wave * KPW + q * 2) * 512);
+    };
+    auto issue_tile = [&](int kt, int stage) {
+#pragma unroll
+        for (int q = 0; q < QN; ++q) {
+            issue_a(kt, stage, q);
+            issue_b(kt, stage, q);
+        }
     };
 
     // ------------------------------------------------------------------------------------------
@@ -357,7 +351,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    bf16x8_t af[2][NI], bfr[2][NJ];
+    bf16x8_t af[NI], bfr[NJ];
     auto read_tr_frag = [&](uint32_t ad, int kk) -> bf16x8_t {
         const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512)));
         const s16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512) + 4 * 512));
@@ -365,25 +359,25 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         return __builtin_bit_cast(bf16x8_t, v);
     };
     // reads the fragments of k sub-step kk from the stage the address registers currently point at
-    auto read_frags = [&](int kk, int buf, auto active) {
+    auto read_frags = [&](int kk, auto active) {
         if (!decltype(active)::value) return;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             if (T::kAKMajor)
-                af[buf][i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(a_ad[i] ^ (uint32_t)(kk << 5));
+                af[i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(a_ad[i] ^ (uint32_t)(kk << 5));
             else
-                af[buf][i] = read_tr_frag(a_ad[i], kk);
+                af[i] = read_tr_frag(a_ad[i], kk);
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             if (T::kBKMajor)
-                bfr[buf][j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(b_ad[j] ^ (uint32_t)(kk << 5));
+                bfr[j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(b_ad[j] ^ (uint32_t)(kk << 5));
             else
-                bfr[buf][j] = read_tr_frag(b_ad[j], kk);
+                bfr[j] = read_tr_frag(b_ad[j], kk);
         }
     };
     // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
-    auto mask_tail = [&](int kt, int kk, int buf) {
+    auto mask_tail = [&](int kt, int kk) {
         if (MODE != kWgrad) return;
         const int valid = tc.rows - kt * BK - kk * 16 - 8 * hi;  // lane holds k = 8*hi + 0..7 of this sub-step
         if (valid >= 8) return;
@@ -395,26 +389,31 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             f = __builtin_bit_cast(bf16x8_t, a);
         };
 #pragma unroll
-        for (int i = 0; i < NI; ++i) zero_tail(af[buf][i]);
+        for (int i = 0; i < NI; ++i) zero_tail(af[i]);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) zero_tail(bfr[buf][j]);
+        for (int j = 0; j < NJ; ++j) zero_tail(bfr[j]);
     };
-    auto mma = [&](int buf, auto active) {
-        if (!decltype(active)::value) return;
+    // The MFMAs of one k-sub-step with side(n) run after MFMA n (n = 0 .. NI*NJ - 1): the slots for this wave's loads.
+    // A wave without rows to compute runs the side jobs alone.
+    auto mma_with = [&](auto active, auto side) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
-            for (int j = 0; j < NJ; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < NJ; ++j) {
+                if (decltype(active)::value)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                side(i * NJ + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
     };
 
     if (n_kt > 0) {
-        issue_loads_part(0, 0, 0, std::false_type{});
-        issue_loads_part(0, 0, 1, std::false_type{});
+        issue_tile(0, 0);
         if (n_kt > 1) {
-            issue_loads_part(1, 1, 0, std::false_type{});
-            issue_loads_part(1, 1, 1, std::false_type{});
+            issue_tile(1, 1);
             // vmcnt(2*QN): tile 0 has landed, tile 1 may still be in flight
+            static_assert(QN == 4 || QN == 8, "wait counts below are written for 4 or 8 loads per operand, wave and k-tile");
             if (QN == 8) __builtin_amdgcn_s_waitcnt(0x4F70);
             else __builtin_amdgcn_s_waitcnt(0x0F78);
         } else {
@@ -422,14 +421,20 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
         __syncthreads();
     }
-    // The k-loop, a ping-pong between two groups of waves.  The eight waves form two groups, one wave of every SIMD in each (waves 0-3 own tile
-    // rows 0..127, waves 4-7 rows 128..255).  A k-sub-step is split into a memory phase (the fragment reads of the
-    // sub-step, some of the operand loads of the next k-tile) and an MFMA phase (its 8 MFMAs back to back), every phase
-    // ends in a barrier, and the second group runs one phase behind the first: while one wave of a SIMD issues MFMAs
-    // the other one reads LDS, and the MFMA pipe goes from one group's 8 MFMAs straight to the other's.  (With both
-    // waves running the same stream, LDS reads and loads interleaved between the MFMAs, the older wave of a SIMD wins
-    // every MFMA slot, reaches the per-k-step barrier early and idles there a third of the time while the younger one
-    // finishes alone: measured with in-kernel cycle counters.)
+    // The k-loop, a ping-pong between two groups of waves.  The eight waves form two groups, one wave of every SIMD in
+    // each (waves 0-3 own tile rows 0..127, waves 4-7 rows 128..255).  A k-sub-step (16 of the 64 k values) is a memory
+    // phase -- the LDS reads of its fragments, in sub-step 3 also the wait for the next k-tile -- followed by an MFMA phase:
+    // its 8 MFMAs, and between them this wave's direct-to-LDS loads of the next k-tile (sub-steps 0 and 1, one load after
+    // every second MFMA) and the L2 prefetch (sub-step 2).  Every phase ends in a barrier and the second group runs one
+    // phase behind the first, so while one wave of a SIMD reads LDS the other owns the MFMA pipe.
+    // Where the loads sit matters.  A vector memory instruction holds its wave for some tens of cycles at issue.  In the
+    // memory phase that time adds to the LDS reads, which alone take about as long as the other group's MFMAs (measured
+    // with a cycle counter at every barrier: memory phases with loads ran 440-470 ticks against 341 for 8 MFMAs, the
+    // ones without 364-400); between two MFMAs it is free, the matrix pipe being busy for 32 cycles per MFMA anyway.
+    // (History of the loop, each step measured side by side in one run: reads, loads and MFMAs interleaved finely in one
+    // stream with two free-running waves per SIMD -- the older wave wins every MFMA slot and then idles a third of the
+    // time at the k-step barrier; ping-pong with the loads in the memory phases, +8 %; loads in the MFMA phases, +4-7 %.)
+    static_assert(NW == 8 && QN == 4, "the load slots of the MFMA phases are laid out for 8 waves (4 loads per operand tile and wave)");
     auto k_loop_pp = [&](auto active) {
         auto phase_end = [&]() {
             __builtin_amdgcn_sched_barrier(0);
@@ -441,49 +446,29 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             const int stage = kt & 1;
             const bool tail = MODE == kWgrad && kt == n_kt - 1;
             const int kt_next = kt + 1 < n_kt ? kt + 1 : n_kt - 1;  // its stage was last read one k-step ago
-            if constexpr (kWidePhases) {
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    // memory phase: the fragments of two sub-steps
-                    read_frags(2 * half, 0, active);
-                    read_frags(2 * half + 1, 1, active);
-                    if (half == 0) {
-                        issue_loads_part(kt_next, stage ^ 1, 0, active);
-                        issue_loads_part(kt_next, stage ^ 1, 1, active);
-                    } else {
-                        prefetch_l2(kt);
-                        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-                        else __builtin_amdgcn_s_waitcnt(0x0F71);
-                    }
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    if (tail) { mask_tail(kt, 2 * half, 0); mask_tail(kt, 2 * half + 1, 1); }
-                    phase_end();
-                    // MFMA phase: 16 MFMAs
-                    mma(0, active);
-                    mma(1, active);
-                    if (half == 1) flip_stage();
-                    phase_end();
+            for (int kk = 0; kk < 4; ++kk) {
+                // memory phase
+                read_frags(kk, active);
+                if (kk == 3) {
+                    // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
+                    if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+                    else __builtin_amdgcn_s_waitcnt(0x0F71);
                 }
-            } else {
-#pragma unroll
-                for (int kk = 0; kk < 4; ++kk) {
-                    // memory phase
-                    read_frags(kk, 0, active);
-                    if (kk < 2) issue_loads_part(kt_next, stage ^ 1, kk, active);
-                    if (kk == 2) prefetch_l2(kt);
-                    if (kk == 3) {
-                        // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
-                        if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-                        else __builtin_amdgcn_s_waitcnt(0x0F71);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (tail) mask_tail(kt, kk);
+                phase_end();
+                // MFMA phase
+                mma_with(active, [&](int n) {
+                    if (kk < 2 && (n & 1) == 0) {
+                        const int q = (QN / 2) * kk + (n >> 2);  // n = 0, 2: loads q of A and B; n = 4, 6: loads q + 1
+                        if ((n & 2) == 0) issue_a(kt_next, stage ^ 1, q);
+                        else issue_b(kt_next, stage ^ 1, q);
                     }
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    if (tail) mask_tail(kt, kk, 0);
-                    phase_end();
-                    // MFMA phase
-                    mma(0, active);
-                    if (kk == 3) flip_stage();
-                    phase_end();
-                }
+                    if (kk == 2 && n == 1) prefetch_l2(kt);
+                });
+                if (kk == 3) flip_stage();
+                phase_end();
             }
         }
         if (wm == 0) phase_end();  // the first group finishes one phase early
