@@ -277,22 +277,24 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         pf_cur += adv;
     };
 
-    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage
+    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage.  The loads are the
+    // opaque form: every wait between a load and the LDS reads of its data is written out in this kernel (prologue,
+    // sub-step 3 of the k-loop, the end of the loop), the compiler adds none.
     auto issue_a = [&](int kt, int stage, int q) {
         char* base = lds + stage * kStageBytes;
         const char* ab = a_base + (int64_t)kt * a_step;
         if (T::kAKMajor)
-            load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
+            load16_to_lds_opaque(ab, a_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds(ab + (uint32_t)(a_off[q] + k_clamp(kt, q) * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(ab, (uint32_t)(a_off[q] + k_clamp(kt, q) * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
     };
     auto issue_b = [&](int kt, int stage, int q) {
         char* base = lds + stage * kStageBytes + kTileBytes;
         const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
         if (T::kBKMajor)
-            load16_to_lds(bb + b_off[q], base + (wave * RPW + q * 8) * 128);
+            load16_to_lds_opaque(bb, b_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds(bb + (uint32_t)(b_off[q] + k_clamp(kt, q) * (int)p.ldb * 2), base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(bb, (uint32_t)(b_off[q] + k_clamp(kt, q) * (int)p.ldb * 2), base + (wave * KPW + q * 2) * 512);
     };
     auto issue_tile = [&](int kt, int stage) {
 #pragma unroll

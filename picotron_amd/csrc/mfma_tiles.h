@@ -21,6 +21,20 @@ __device__ __forceinline__ void load16_to_lds(const void* g, char* l) {
                                      (__attribute__((address_space(3))) void*)l, 16, 0, 0);
 }
 
+// The same load as an instruction sequence the compiler does not look into: wave-uniform base pointer plus a 32-bit
+// byte offset per lane, LDS destination (wave-uniform, lane l lands at +16*l) through M0.  Why: the compiler's
+// wait-count pass knows a builtin direct-to-LDS load is in flight and puts "s_waitcnt vmcnt(0)" in front of every later
+// LDS read it cannot prove disjoint from the destination -- it does so for the transpose reads
+// (__builtin_amdgcn_ds_read_tr16_b64), which then wait for loads issued a moment ago.  A kernel that uses this form
+// orders its LDS reads after the loads itself (explicit s_waitcnt vmcnt + barrier).  M0 is written here and is not in the
+// clobber list (the compiler rejects it as reserved): nothing else in a kernel that uses this form may depend on M0 --
+// no builtin direct-to-LDS load, no s_sendmsg, no GWS.
+__device__ __forceinline__ void load16_to_lds_opaque(const char* base, uint32_t lane_offset, char* l) {
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)l;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(lane_offset), "s"(base) : "memory");
+}
+
 
 __device__ __forceinline__ int uniform_i32(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ int64_t uniform_i64(int64_t v) {
