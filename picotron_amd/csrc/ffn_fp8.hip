@@ -61,14 +61,19 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
         a_off[q] = (uint32_t)(ar * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
         b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
     }
-    auto issue_loads = [&](int kt, int stage, int q0) {  // half of a wave's loads for one k-tile
-        char* base = lds + stage * kStageBytes;
-        const char* ab = a_base + (int64_t)kt * kFp8BK;
-        const char* bb = b_base + (int64_t)kt * kFp8BK;
+    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt.  Opaque loads: the waits between
+    // a load and the LDS reads of its data are the explicit ones below (prologue, k-loop barrier, end of the loop).
+    auto issue_a = [&](int kt, int stage, int q) {
+        load16_to_lds_opaque(a_base + (int64_t)kt * kFp8BK, a_off[q], lds + stage * kStageBytes + (wave * RPW + q * 8) * 128);
+    };
+    auto issue_b = [&](int kt, int stage, int q) {
+        load16_to_lds_opaque(b_base + (int64_t)kt * kFp8BK, b_off[q], lds + stage * kStageBytes + kTileBytes + (wave * RPW + q * 8) * 128);
+    };
+    auto issue_tile = [&](int kt, int stage) {
 #pragma unroll
-        for (int q = q0; q < q0 + QN / 2; ++q) {
-            load16_to_lds(ab + a_off[q], base + (wave * RPW + q * 8) * 128);
-            load16_to_lds(bb + b_off[q], base + kTileBytes + (wave * RPW + q * 8) * 128);
+        for (int q = 0; q < QN; ++q) {
+            issue_a(kt, stage, q);
+            issue_b(kt, stage, q);
         }
     };
 
@@ -110,68 +115,67 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     i32x8_t af[2][NI], bfr[2][NJ];
-    auto read_frags = [&](int s, int buf, auto active) {
-        if (!decltype(active)::value) return;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) af[buf][i] = read_frag(a_ad[i], s);
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) bfr[buf][j] = read_frag(b_ad[j], s);
+    // fragment f of sub-step sub into buffer buf: f = 0..3 the A row blocks, 4..5 the B column blocks
+    auto read_one = [&](int f, int sub, int buf) {
+        if (f < NI) af[buf][f] = read_frag(a_ad[f], sub);
+        else bfr[buf][f - NI] = read_frag(b_ad[f - NI], sub);
     };
-    auto mma = [&](int buf, auto active) {
-        if (!decltype(active)::value) return;
+    // the 8 MFMAs (64 cycles each) of one sub-step with side(n) run after MFMA n: the slots for LDS reads and loads
+    auto mma_with = [&](int buf, auto active, auto side) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
-            for (int j = 0; j < NJ; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+            for (int j = 0; j < NJ; ++j) {
+                if (decltype(active)::value)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                side(i * NJ + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
     };
-    // one sub-step: 8 MFMAs (64 cycles each), the 12 LDS reads of the next sub-step and 4 direct-to-LDS loads,
-    // spread one MFMA : two reads : one load over the first MFMAs
-#define PICOMOE_FP8_INTERLEAVE()                                  \
-    _Pragma("unroll") for (int s_ = 0; s_ < 6; ++s_) {            \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);        \
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        \
-    }                                                             \
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
 
     if (n_kt > 0) {
-        issue_loads(0, 0, 0);
-        issue_loads(0, 0, QN / 2);
+        issue_tile(0, 0);
         if (n_kt > 1) {
-            issue_loads(1, 1, 0);
-            issue_loads(1, 1, QN / 2);
+            issue_tile(1, 1);
             __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): tile 0 has landed, tile 1 may still be in flight
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         __syncthreads();
-        if (wave_active) read_frags(0, 0, std::true_type{});
+        if (wave_active) {
+#pragma unroll
+            for (int f = 0; f < NI + NJ; ++f) read_one(f, 0, 0);
+        }
     }
+    // One k-step = two sub-steps.  Sub-step 0: its MFMAs with the fragment reads of sub-step 1 between them; then every
+    // wave holds its last fragments of this stage in registers, waits for its loads of the next k-tile (issued a whole
+    // k-step ago) and meets the others at the barrier.  Sub-step 1: its MFMAs with all 8 loads of k-tile kt+2 into the
+    // stage just vacated, two after each of the first four MFMAs (issued right after the barrier they have the longest
+    // time to land: split 4 + 4 around the barrier the kernel was 4.5 % slower, one per MFMA 2 % slower), and the fragment
+    // reads of sub-step 0 of k-tile kt+1 from the other stage after MFMAs 2..7.
     auto k_loop = [&](auto active) {
+        constexpr bool kActive = decltype(active)::value;
         for (int kt = 0; kt < n_kt; ++kt) {
             const int stage = kt & 1;
-            __builtin_amdgcn_sched_barrier(0);
-            // second half of the refill begun in the previous k-step (clamped past the end: lands in a dead stage)
-            issue_loads(kt + 1 < n_kt ? kt + 1 : n_kt - 1, stage ^ 1, QN / 2);
-            read_frags(1, 1, active);
-            mma(0, active);
-            PICOMOE_FP8_INTERLEAVE()
-            __builtin_amdgcn_sched_barrier(0);
-            // every wave holds its last fragments of this stage in registers and the next tile has landed
+            const int kt_load = kt + 2 < n_kt ? kt + 2 : n_kt - 1;  // clamped past the end: lands in a dead stage
+            mma_with(0, active, [&](int n) {
+                if (kActive && n < NI + NJ) read_one(n, 1, 1);
+            });
             __builtin_amdgcn_s_waitcnt(0x0F70);
-            __syncthreads();
-            issue_loads(kt + 2 < n_kt ? kt + 2 : n_kt - 1, stage, 0);
-            flip_stage();
-            read_frags(0, 0, active);  // past the last tile this reads a stage that is not used any more
-            mma(1, active);
-            PICOMOE_FP8_INTERLEAVE()
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            flip_stage();
+            mma_with(1, active, [&](int n) {
+                if (n < 4) { issue_a(kt_load, stage, n); issue_b(kt_load, stage, n); }
+                if (kActive && n >= 2) read_one(n - 2, 0, 0);  // past the last tile this reads a stage that is not used any more
+            });
         }
     };
     if (wave_active) k_loop(std::true_type{});
     else k_loop(std::false_type{});
-#undef PICOMOE_FP8_INTERLEAVE
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
