@@ -40,6 +40,9 @@ constexpr int kWaves = PICOMOE_MFMA_WAVES;
 #define PICOMOE_PREFETCH_BWD 2
 #endif
 
+#ifndef PICOMOE_ROW_BLOCK_SKIP
+#define PICOMOE_ROW_BLOCK_SKIP 1
+#endif
 enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
 
 template <int MODE>
@@ -139,7 +142,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
     // a wavefront whose 128 rows all lie past the end of the expert's segment keeps loading and synchronising
     // but skips its fragment reads and MFMAs
-    const bool wave_active = MODE == kWgrad || wm * 128 < tc.rows;
+    // 32-row blocks of this wave's 128 rows that hold rows of the expert's segment (wgrad: all four; its ragged dimension is K)
+    const int rows_here = MODE == kWgrad ? 128 : (tc.rows - wm * 128 < 0 ? 0 : (tc.rows - wm * 128 > 128 ? 128 : tc.rows - wm * 128));
+    const int active_blocks = (rows_here + 31) / 32;
 
     // ------------------------------------------------------------------------------------------
     // global -> LDS: a wave-uniform base pointer per operand plus, per lane, a 32-bit byte offset for each
@@ -362,9 +367,10 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     };
     // reads the fragments of k sub-step kk from the stage the address registers currently point at
     auto read_frags = [&](int kk, auto active) {
-        if (!decltype(active)::value) return;
+        constexpr int kActiveBlocks = decltype(active)::value;
+        if (kActiveBlocks == 0) return;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < kActiveBlocks; ++i) {
             if (T::kAKMajor)
                 af[i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(a_ad[i] ^ (uint32_t)(kk << 5));
             else
@@ -396,13 +402,13 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         for (int j = 0; j < NJ; ++j) zero_tail(bfr[j]);
     };
     // The MFMAs of one k-sub-step with side(n) run after MFMA n (n = 0 .. NI*NJ - 1): the slots for this wave's loads.
-    // A wave without rows to compute runs the side jobs alone.
+    // `active` carries the number of 32-row blocks the wave computes; a wave without rows runs the side jobs alone.
     auto mma_with = [&](auto active, auto side) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                if (decltype(active)::value)
+                if (i < decltype(active)::value)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 side(i * NJ + j);
@@ -475,10 +481,17 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
         if (wm == 0) phase_end();  // the first group finishes one phase early
     };
-    // Two copies of the loop, picked per wave: waves that own rows of the tile run all of it; a wave whose 128 rows lie
-    // past the end of a short tail only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).
-    if (wave_active) k_loop_pp(std::true_type{});
-    else k_loop_pp(std::false_type{});
+    // Five copies of the loop, picked per wave by the number of its 32-row blocks that hold rows of the segment: a wave
+    // reads A fragments and issues MFMAs for those blocks only, and one whose 128 rows all lie past the end of a short tail
+    // only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).  A tail tile then costs about what
+    // its rows are worth instead of a half or a whole tile.
+    switch (PICOMOE_ROW_BLOCK_SKIP ? active_blocks : (active_blocks > 0 ? 4 : 0)) {
+        case 4: k_loop_pp(std::integral_constant<int, 4>{}); break;
+        case 3: k_loop_pp(std::integral_constant<int, 3>{}); break;
+        case 2: k_loop_pp(std::integral_constant<int, 2>{}); break;
+        case 1: k_loop_pp(std::integral_constant<int, 1>{}); break;
+        default: k_loop_pp(std::integral_constant<int, 0>{}); break;
+    }
     // the clamped refills of the last k-steps may still be landing in LDS, which the epilogue reuses
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -532,6 +545,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
+            if (wm * 128 + i * 32 >= valid_rows) continue;  // wave-uniform: a block of rows past the segment has nothing to store
             // g and u rounded to bf16 in place (what the reference's two Linear outputs hold)
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
@@ -553,6 +567,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
+            if (wm * 128 + i * 32 >= valid_rows) continue;
             stage_block([&](int j, int r) { return acc[i][j][r]; });
             for_chunks(i, [&](int trow, int c, u32x4_t v) {
                 const int64_t col = col0 + c;
