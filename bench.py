@@ -31,7 +31,7 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # L2 <-> memory bytes of the grouped-GEMM launches of one layer step, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE x 2 KiB, WRITE_SIZE x 1 KiB; factors from the --traffic-probe copy kernel).  Algorithmic: 15.5e9.
-MEASURED_TRAFFIC_BYTES = {"c5": 36.1e9}
+MEASURED_TRAFFIC_BYTES = {"c5": 35.2e9}
 
 WORKLOADS = {
     # name: tokens, hidden, ffn, experts, top_k, shared, capacity_factor, fp8_dispatch, backward
