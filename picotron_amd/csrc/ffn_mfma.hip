@@ -216,11 +216,19 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     }
     // wgrad: k rows past the expert's last row are re-read from its last row and masked out of the fragments
-    auto k_clamp = [&](int kt, int q) -> int {
-        if (MODE != kWgrad) return 0;
-        const int kr = kt * BK + wave * KPW + q * 2 + (lane >> 5);
-        return kr < tc.rows ? 0 : tc.rows - 1 - kr;
-    };
+    // Only the last k-tile can reach past the segment, so its clamped lane offsets are worked out once, here, and a
+    // load picks between the two precomputed offsets with one select (computing the clamp at every load put a dependent
+    // chain of vector instructions, a 64-bit multiply-add among them, between the MFMAs of wgrad's load phases).
+    uint32_t a_off_tail[T::kAKMajor ? 1 : QN], b_off_tail[T::kBKMajor ? 1 : QN];
+    if (MODE == kWgrad) {
+#pragma unroll
+        for (int q = 0; q < QN; ++q) {
+            const int kr = (n_kt - 1) * BK + wave * KPW + q * 2 + (lane >> 5);
+            const int dk = kr < tc.rows ? 0 : tc.rows - 1 - kr;
+            if (!T::kAKMajor) a_off_tail[q] = (uint32_t)((int)a_off[q] + dk * (int)p.lda * 2);
+            if (!T::kBKMajor) b_off_tail[q] = (uint32_t)((int)b_off[q] + dk * (int)p.ldb * 2);
+        }
+    }
     // ------------------------------------------------------------------------------------------
     // L2 prefetch.  The demand loads of the blocks that share an operand slice reach the L2 together, and when the
     // slice still has to come from HBM they all queue behind the same misses.  So every k-step each wave touches
@@ -291,7 +299,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         if (T::kAKMajor)
             load16_to_lds_opaque(ab, a_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds_opaque(ab, (uint32_t)(a_off[q] + k_clamp(kt, q) * (int)p.lda * 2), base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(ab, MODE == kWgrad && kt == n_kt - 1 ? a_off_tail[q] : a_off[q], base + (wave * KPW + q * 2) * 512);
     };
     auto issue_b = [&](int kt, int stage, int q) {
         char* base = lds + stage * kStageBytes + kTileBytes;
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         if (T::kBKMajor)
             load16_to_lds_opaque(bb, b_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds_opaque(bb, (uint32_t)(b_off[q] + k_clamp(kt, q) * (int)p.ldb * 2), base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(bb, MODE == kWgrad && kt == n_kt - 1 ? b_off_tail[q] : b_off[q], base + (wave * KPW + q * 2) * 512);
     };
     auto issue_tile = [&](int kt, int stage) {
 #pragma unroll
