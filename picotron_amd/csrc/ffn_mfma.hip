@@ -586,18 +586,20 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                     const u32x4_t gv = *(const u32x4_t*)(p.aux + grow * 2 * I + col);
                     const u32x4_t uv = *(const u32x4_t*)(p.aux + grow * 2 * I + I + col);
                     u32x4_t dgv, duv, av;
+                    const bool want_act = p.out2 != nullptr;  // the recomputed activation is only worked out when asked for
 #pragma unroll
                     for (int w2 = 0; w2 < 4; ++w2) {
-                        float o_dg[2], o_du[2], o_a[2];
+                        float o_dg[2], o_du[2], o_a[2] = {0.f, 0.f};
 #pragma unroll
                         for (int h2 = 0; h2 < 2; ++h2) {
                             const float da = __uint_as_float(h2 ? (v[w2] & 0xFFFF0000u) : (v[w2] << 16));
                             const float g = __uint_as_float(h2 ? (gv[w2] & 0xFFFF0000u) : (gv[w2] << 16));
                             const float u = __uint_as_float(h2 ? (uv[w2] & 0xFFFF0000u) : (uv[w2] << 16));
                             const float sig = sigmoid_fast(g);
-                            o_dg[h2] = da * u * (sig * (1.f + g * (1.f - sig)));
-                            o_du[h2] = da * (g * sig);
-                            o_a[h2] = bf16_bits_to_f32(f32_to_bf16_bits(g * sig)) * u;
+                            const float gs = g * sig;
+                            o_dg[h2] = da * u * (sig + gs * (1.f - sig));
+                            o_du[h2] = da * gs;
+                            if (want_act) o_a[h2] = bf16_bits_to_f32(f32_to_bf16_bits(gs)) * u;
                         }
                         dgv[w2] = pack_bf16x2(o_dg[0], o_dg[1]);
                         duv[w2] = pack_bf16x2(o_du[0], o_du[1]);
@@ -605,7 +607,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                     }
                     *(u32x4_t*)(p.out + grow * 2 * I + col) = dgv;
                     *(u32x4_t*)(p.out + grow * 2 * I + I + col) = duv;
-                    if (p.out2) *(u32x4_t*)(p.out2 + grow * I + col) = av;
+                    if (want_act) *(u32x4_t*)(p.out2 + grow * I + col) = av;
                 } else if (MODE == kDown && p.aux) {
                     const float rw = bf16_bits_to_f32(p.aux[grow]);
                     u32x4_t o;
