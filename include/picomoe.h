@@ -27,7 +27,7 @@ extern "C" {
 #define PICOMOE_F32 0
 #define PICOMOE_BF16 1
 
-#define PICOMOE_ABI_VERSION 1
+#define PICOMOE_ABI_VERSION 2
 
 /* ABI version of the loaded library (compare with PICOMOE_ABI_VERSION). */
 int picomoe_abi_version(void);
@@ -127,7 +127,8 @@ int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, const int64_t*
                             const float* up_scale, void* act, void* inter13, void* stream);
 /* Replaces the down grouped GEMM with its optional row-weight epilogue (EP/megakernel.py:305, :95-96). */
 int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden, int64_t inter,
-                     const void* down_w, const void* row_weight, int dtype, void* y, void* stream);
+                     const void* down_w, const void* row_weight, int dtype, void* y, void* workspace, int64_t workspace_bytes,
+                     void* stream);
 /* Replaces da = dy @ down_w[e] and _silu_and_mul_bwd (EP/megakernel.py:344-345, :187-197) in one kernel:
  * d_inter13 [n_rows, 2*inter] = [dg | du]; act_out (optional) = silu(g) * u rebuilt from inter13. */
 int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
@@ -135,7 +136,15 @@ int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts
                           void* stream);
 /* Replaces dx = d_inter13 @ w13[e] (EP/megakernel.py:346) without the concatenated w13. */
 int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
-                        int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx, void* stream);
+                        int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+/* Device scratch the two calls above can use (the library allocates nothing itself, the boundary rule of the reference's
+ * kernels being torch-owned memory: EP/megakernel.py:294-306 allocates every buffer with torch.empty).  With
+ * `workspace` of at least this many bytes the bf16 kernels cut the tiles of the last, partly filled round of blocks into
+ * 2 or 4 ranges of K that run side by side, park the fp32 partial tiles there and add them up in a second small kernel;
+ * with NULL (or fewer bytes) every tile is computed whole.  Results agree to the rounding of the fp32 partial sums.
+ * Calls that overlap in time on different streams need a workspace each. */
+int64_t picomoe_ffn_workspace_bytes(void);
 /* Replaces _grouped_wgrad (EP/megakernel.py:209-291): out [E, p_dim, q_dim] with out[e] = lhs_e^T @ rhs_e over the
  * rows of expert e; lhs [n_rows, >=p_dim] with row stride ld_lhs, rhs likewise (so the two halves of d_inter13
  * are addressed in place).  Empty experts get zeros. */

@@ -34,13 +34,16 @@ extern "C" int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, con
     return ffn_fp8_gate_up(s, xq, x_scale, gate_wq, up_wq, gate_scale, up_scale, act, inter13, (hipStream_t)stream);
 }
 
+extern "C" int64_t picomoe_ffn_workspace_bytes(void) { return ffn_mfma_workspace_bytes(); }
+
 extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
-                                int64_t inter, const void* down_w, const void* row_weight, int dtype, void* y, void* stream) {
+                                int64_t inter, const void* down_w, const void* row_weight, int dtype, void* y, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
     FfnShape s;
     PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(act && down_w && y);
-    if (ffn_mfma_supported(s)) return ffn_mfma_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
+    if (ffn_mfma_supported(s)) return ffn_mfma_down(s, act, down_w, row_weight, y, workspace, workspace_bytes, (hipStream_t)stream);
     return ffn_simple_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
 }
 
@@ -57,12 +60,12 @@ extern "C" int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int 
 
 extern "C" int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_experts, int64_t n_rows,
                                    int64_t hidden, int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx,
-                                   void* stream) {
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
     FfnShape s;
     PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(d_inter13 && gate_w && up_w && dx);
-    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
+    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_x(s, d_inter13, gate_w, up_w, dx, workspace, workspace_bytes, (hipStream_t)stream);
     return ffn_simple_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
 }
 

@@ -70,6 +70,8 @@ struct MfmaParams {
     int64_t ldo;
     uint16_t* out2;       // gate/up: inter13 (optional); dgrad_act: act_out (optional)
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
+    float* ws;            // down, dgrad_x: fp32 partial tiles of the split last round (kSplitWorkspaceBytes), or null
+    int max_pieces;       // 1 = no split
 };
 
 // X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
@@ -128,18 +130,22 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     constexpr int RPW = QN * 8;         // K-major tile rows a wave fills
     constexpr int KPW = QN * 2;         // X-major k rows a wave fills
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
+    constexpr bool kCanSplit = MODE == kDown || MODE == kDgradX;
     TileCoord tc;
     if (MODE == kWgrad) {
         if (!locate_wgrad(p.counts, p.E, p.m_tiles, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
     } else {
-        if (!locate_m_grouped(p.counts, p.E, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
+        if (!locate_m_grouped(p.counts, p.E, p.n_tiles, blockIdx.x / kNumXcd, &tc, kCanSplit ? p.max_pieces : 1)) return;
     }
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS bases and row ranges stay scalar
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
     const int l31 = lane & 31, hi = lane >> 5;
-    const int n_kt = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
+    // k-tiles of this block: all of K, or this piece's share of it
+    const int n_kt_all = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
+    const int kt_first = kCanSplit ? (int)((int64_t)tc.piece * n_kt_all / tc.pieces) : 0;
+    const int n_kt = kCanSplit ? (int)((int64_t)(tc.piece + 1) * n_kt_all / tc.pieces) - kt_first : n_kt_all;
     // a wavefront whose 128 rows all lie past the end of the expert's segment keeps loading and synchronising
     // but skips its fragment reads and MFMAs
     // 32-row blocks of this wave's 128 rows that hold rows of the expert's segment (wgrad: all four; its ragged dimension is K)
@@ -156,6 +162,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     int64_t a_step, b_step;      // bytes per k-tile
     int64_t b_switch_delta = 0;  // dgrad_x: jump from gate_w to up_w half way through K
     int b_switch_kt = 0x7FFFFFFF;
+    int64_t b_jump_now = 0;      // dgrad_x, a piece that starts in the up_w half: the same jump, taken from the start
     if (T::kAKMajor) {
         // wave w fills tile rows [RPW*w, RPW*(w+1)), 8 rows (128 B each) per instruction
         a_step = BK * 2;
@@ -203,8 +210,16 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         b_step = BK * p.ldb * 2;
         b_base = (const char*)(MODE == kWgrad ? p.B0 + tc.row0 * p.ldb : p.B0 + (int64_t)tc.e * p.b_expert_stride);
         if (MODE == kDgradX) {
-            b_switch_kt = n_kt / 2;
-            b_switch_delta = ((const char*)p.B1 - (const char*)p.B0) - (int64_t)b_switch_kt * b_step;
+            // B moves from gate_w to up_w at k-tile n_kt_all / 2 of the whole K; in this block's own numbering
+            // (k-tile 0 = kt_first) that is either still ahead or already behind
+            const int sw = n_kt_all / 2;
+            const int64_t jump = ((const char*)p.B1 - (const char*)p.B0) - (int64_t)sw * b_step;
+            if (kt_first >= sw) {
+                b_jump_now = jump;
+            } else if (sw - kt_first < n_kt) {  // a piece that ends at or before the switch never takes the jump
+                b_switch_kt = sw - kt_first;
+                b_switch_delta = jump;
+            }
         }
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
@@ -216,6 +231,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     }
     // wgrad: k rows past the expert's last row are re-read from its last row and masked out of the fragments
+    a_base += (int64_t)kt_first * a_step;
+    b_base += (int64_t)kt_first * b_step + b_jump_now;
     // Only the last k-tile can reach past the segment, so its clamped lane offsets are worked out once, here, and a
     // load picks between the two precomputed offsets with one select (computing the clamp at every load put a dependent
     // chain of vector instructions, a 64-bit multiply-add among them, between the MFMAs of wgrad's load phases).
@@ -273,6 +290,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             }
         }
     }
+    pf_ptr += (int64_t)kt_first * pf_step + (wave >= NW / 2 ? b_jump_now : 0);
     const int64_t pf_switch_delta = wave >= NW / 2 ? b_switch_delta : 0;
     // wgrad: only k-tiles that lie completely inside the expert's rows are prefetched
     const int pf_n_kt = MODE == kWgrad ? tc.rows / BK : n_kt;
@@ -511,6 +529,21 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // the last barrier) and reads them back row-contiguously, so HBM sees 16-byte lanes and 128..256-byte
     // row segments, and the fused SwiGLU backward reads g / u the same way.
     // ------------------------------------------------------------------------------------------
+    if (kCanSplit && tc.pieces > 1) {
+        // a piece of a split tile: the fp32 accumulators go to the workspace as they are; ffn_mfma_fixup_kernel adds the
+        // pieces up in a fixed order and applies the epilogue
+        float* w = p.ws + (int64_t)tc.ws_slot * (BM * BN);
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+                    if (row < tc.rows) w[row * BN + wn * CW + j * 32 + l31] = acc[i][j][r];
+                }
+        return;
+    }
     int valid_rows = tc.rows;
     int64_t out_row0 = tc.row0;
     if (MODE == kWgrad) {
@@ -623,15 +656,55 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     }
 }
 
+// Second pass of a split last round: block b adds up the fp32 pieces of remainder tile b / 8 of XCD b % 8 (in piece
+// order, so the result does not depend on timing) and applies the epilogue of the unsplit kernel: accumulators rounded to
+// the output type; down: times the row weight, rounded again.
+template <int MODE>
+__global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
+    const GroupedLayout g = grouped_layout(p.counts, p.E, p.n_tiles, p.max_pieces);
+    const int t = blockIdx.x / kNumXcd, xcd = blockIdx.x % kNumXcd;
+    if (g.pieces <= 1 || t >= g.rem) return;
+    TileCoord tc;
+    if (!locate_tile_slot(p.counts, p.E, p.n_tiles, g, xcd, g.full + t, &tc)) return;
+    const float* w = p.ws + (int64_t)(xcd * kCusPerXcd + t * g.pieces) * (BM * BN);
+    const int c4 = (threadIdx.x & 63) * 4;
+    for (int row = threadIdx.x >> 6; row < tc.rows; row += 4) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        for (int pc = 0; pc < g.pieces; ++pc) {
+            const f32x4_t v = *(const f32x4_t*)(w + (int64_t)pc * (BM * BN) + row * BN + c4);
+            s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+        }
+        s0 = bf16_bits_to_f32(f32_to_bf16_bits(s0)); s1 = bf16_bits_to_f32(f32_to_bf16_bits(s1));
+        s2 = bf16_bits_to_f32(f32_to_bf16_bits(s2)); s3 = bf16_bits_to_f32(f32_to_bf16_bits(s3));
+        const int64_t grow = tc.row0 + row;
+        if (MODE == kDown && p.aux) {
+            const float rw = bf16_bits_to_f32(p.aux[grow]);
+            s0 *= rw; s1 *= rw; s2 *= rw; s3 *= rw;
+        }
+        uint32_t o[2] = {pack_bf16x2(s0, s1), pack_bf16x2(s2, s3)};
+        *(uint64_t*)(p.out + grow * p.ldo + (int64_t)tc.n_tile * BN + c4) = (uint64_t)o[0] | ((uint64_t)o[1] << 32);
+    }
+}
+
+// how many pieces the tiles of the last round may be cut into: none without the workspace, and none below 16 k-tiles a piece
+int split_pieces(const void* ws, int64_t ws_bytes, int64_t k_tiles) {
+    if (!ws || ws_bytes < kSplitWorkspaceBytes) return 1;
+    const int64_t by_k = k_tiles / 16;
+    return by_k >= kMaxSplit ? kMaxSplit : (by_k >= 2 ? 2 : 1);
+}
+
 MfmaParams base_params(const FfnShape& s) {
     MfmaParams p{};
     p.counts = s.counts;
     p.E = s.E;
     p.n_rows = s.n_rows;
+    p.max_pieces = 1;
     return p;
 }
 
 }  // namespace
+
+int64_t ffn_mfma_workspace_bytes() { return kSplitWorkspaceBytes; }
 
 bool ffn_mfma_supported(const FfnShape& s) {
     return s.dtype == PICOMOE_BF16 && s.H % 256 == 0 && s.I % 128 == 0 && s.H >= 256 && s.I >= 128;
@@ -648,13 +721,17 @@ int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const
     return picomoe_launch_status();
 }
 
-int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, hipStream_t st) {
+int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, void* ws,
+                  int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
     p.K = s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
     p.A = (const uint16_t*)act; p.lda = s.I;
     p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;
     p.out = (uint16_t*)y; p.ldo = s.H; p.aux = (const uint16_t*)row_weight;
-    hipLaunchKernelGGL((ffn_mfma_kernel<kDown, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
+    p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDown, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
+    if (p.max_pieces > 1)
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDown>), dim3(kNumXcd * (kCusPerXcd / 2)), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -669,14 +746,17 @@ int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, co
     return picomoe_launch_status();
 }
 
-int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx,
-                     hipStream_t st) {
+int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx, void* ws,
+                     int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
     p.K = 2 * s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
     p.A = (const uint16_t*)d_inter13; p.lda = 2 * s.I;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;  // [K = I][N = H]
     p.out = (uint16_t*)dx; p.ldo = s.H;
-    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradX, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
+    p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradX, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
+    if (p.max_pieces > 1)
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDgradX>), dim3(kNumXcd * (kCusPerXcd / 2)), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 

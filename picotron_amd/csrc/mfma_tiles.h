@@ -49,6 +49,9 @@ struct TileCoord {
     // L2 prefetch shares: of the tiles one XCD runs at a time, a_sn share this tile's A slices and b_sn its B slices;
     // this tile touches lines a_si, a_si + a_sn, ... of an A slice and b_si, b_si + b_sn, ... of a B slice
     int a_si, a_sn, b_si, b_sn;
+    // split last round (M-grouped kernels that are given a workspace): this block computes k range `piece` of `pieces`
+    // and leaves its fp32 partial tile in workspace slot ws_slot
+    int piece, pieces, ws_slot;
 };
 
 
@@ -71,10 +74,24 @@ __device__ __forceinline__ int wave_scan_i32(int v, int lane) {  // inclusive pr
     return v;
 }
 
-// The lookup runs in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[] per pass instead
-// of a chain of dependent scalar loads.  Tile and row totals fit 32 bits.  `slot` is the position of the wanted tile
-// in this block's XCD's run of tiles (blockIdx.x / 8).
-__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, int64_t slot, TileCoord* tc) {
+constexpr int kCusPerXcd = 32;
+constexpr int kMaxSplit = 4;
+// fp32 partial tiles of the split last round: at most kCusPerXcd pieces per XCD
+constexpr int64_t kSplitWorkspaceBytes = (int64_t)kNumXcd * kCusPerXcd * BM * BN * 4;
+
+// How the M-grouped tiles of a launch are laid out over the XCDs: every XCD runs `heavy_per_xcd` heavy tiles and then
+// `light_per_xcd` light ones (slots 0 .. per_xcd - 1).  With max_pieces > 1, the tiles left over after the full rounds of
+// kCusPerXcd (`rem` of them, slots >= full) are cut into `pieces` ranges of K each, so that the last, partly filled round
+// takes 1 / pieces of a tile instead of a whole one: slot full + t * pieces + p is piece p of tile slot full + t.
+struct GroupedLayout {
+    int64_t heavy, light, heavy_per_xcd, light_per_xcd, per_xcd;
+    int64_t full;  // slots of whole tiles that come first
+    int rem, pieces;
+};
+
+// Runs in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[] per pass instead of a chain
+// of dependent scalar loads.  Tile and row totals fit 32 bits.
+__device__ __forceinline__ GroupedLayout grouped_layout(const int64_t* counts, int E, int n_tiles, int max_pieces) {
     const int lane = threadIdx.x & 63;
     int heavy_m = 0, light_m = 0;
     for (int base = 0; base < E; base += 64) {
@@ -84,19 +101,43 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
     }
     heavy_m = uniform_i32(wave_sum_i32(heavy_m));  // the same in every lane: scalar from here on
     light_m = uniform_i32(wave_sum_i32(light_m));
-    const int64_t heavy = (int64_t)heavy_m * n_tiles, light = (int64_t)light_m * n_tiles;
-    const int64_t heavy_per_xcd = (heavy + kNumXcd - 1) / kNumXcd, light_per_xcd = (light + kNumXcd - 1) / kNumXcd;
-    const int64_t xcd = blockIdx.x % kNumXcd;
+    GroupedLayout g;
+    g.heavy = (int64_t)heavy_m * n_tiles;
+    g.light = (int64_t)light_m * n_tiles;
+    g.heavy_per_xcd = (g.heavy + kNumXcd - 1) / kNumXcd;
+    g.light_per_xcd = (g.light + kNumXcd - 1) / kNumXcd;
+    g.per_xcd = g.heavy_per_xcd + g.light_per_xcd;
+    g.full = g.per_xcd;
+    g.rem = 0;
+    g.pieces = 1;
+    if (max_pieces > 1) {
+        const int rem = (int)(g.per_xcd % kCusPerXcd);
+        int pieces = rem == 0 ? 1 : kCusPerXcd / rem;
+        if (pieces > max_pieces) pieces = max_pieces;
+        if (pieces == 3) pieces = 2;
+        if (pieces > 1) {
+            g.full = g.per_xcd - rem;
+            g.rem = rem;
+            g.pieces = pieces;
+        }
+    }
+    return g;
+}
+
+// Tile number `tile_slot` (0 .. per_xcd - 1) of XCD `xcd`.
+__device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, int n_tiles, const GroupedLayout& g, int64_t xcd,
+                                                 int64_t tile_slot, TileCoord* tc) {
+    const int lane = threadIdx.x & 63;
     bool want_light;
     int64_t L;
-    if (slot < heavy_per_xcd) {
+    if (tile_slot < g.heavy_per_xcd) {
         want_light = false;
-        L = xcd * heavy_per_xcd + slot;
-        if (L >= heavy) return false;
-    } else if (slot - heavy_per_xcd < light_per_xcd) {
+        L = xcd * g.heavy_per_xcd + tile_slot;
+        if (L >= g.heavy) return false;
+    } else if (tile_slot < g.per_xcd) {
         want_light = true;
-        L = xcd * light_per_xcd + (slot - heavy_per_xcd);
-        if (L >= light) return false;
+        L = xcd * g.light_per_xcd + (tile_slot - g.heavy_per_xcd);
+        if (L >= g.light) return false;
     } else {
         return false;
     }
@@ -133,6 +174,25 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
     return false;
 }
 
+// The tile (and, with max_pieces > 1, the piece of it) behind position `slot` of this block's XCD's run (blockIdx.x / 8).
+__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, int64_t slot, TileCoord* tc,
+                                                 int max_pieces = 1) {
+    const GroupedLayout g = grouped_layout(counts, E, n_tiles, max_pieces);
+    int64_t tile_slot = slot;
+    tc->piece = 0;
+    tc->pieces = 1;
+    tc->ws_slot = 0;
+    if (slot >= g.full && g.pieces > 1) {
+        const int64_t idx = slot - g.full;
+        if (idx >= (int64_t)g.rem * g.pieces) return false;
+        tile_slot = g.full + idx / g.pieces;
+        tc->piece = (int)(idx % g.pieces);
+        tc->pieces = g.pieces;
+        tc->ws_slot = (int)((blockIdx.x % kNumXcd) * kCusPerXcd + idx);
+    }
+    return locate_tile_slot(counts, E, n_tiles, g, blockIdx.x % kNumXcd, tile_slot, tc);
+}
+
 // first row of expert e's segment: the sum of the counts before it
 __device__ __forceinline__ int64_t segment_start(const int64_t* counts, int e) {
     const int lane = threadIdx.x & 63;
@@ -144,8 +204,9 @@ __device__ __forceinline__ int64_t segment_start(const int64_t* counts, int e) {
 
 inline unsigned round_up_xcd(int64_t g) { return (unsigned)(((g + kNumXcd - 1) / kNumXcd) * kNumXcd); }
 // upper bound of 8 * (ceil(heavy / 8) + ceil(light / 8)) over every split of the rows among the experts
-inline unsigned grid_m_grouped(const FfnShape& s, int n_tiles) {
-    return round_up_xcd((s.n_rows / BM + s.E) * (int64_t)n_tiles) + 2 * kNumXcd;
+inline unsigned grid_m_grouped(const FfnShape& s, int n_tiles, bool split = false) {
+    // a split last round adds at most kCusPerXcd slots per XCD
+    return round_up_xcd((s.n_rows / BM + s.E) * (int64_t)n_tiles) + 2 * kNumXcd + (split ? kNumXcd * kCusPerXcd : 0);
 }
 
 

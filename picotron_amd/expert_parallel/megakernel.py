@@ -92,14 +92,30 @@ def _gate_up_fp8(xq, x_scale, counts, gate_q, gate_scale, up_q, up_scale, keep_i
     return act, inter13
 
 
+_workspaces = {}
+
+
+def _ffn_workspace(device):
+    """Scratch for the split last round of the down / dgrad_x kernels (picomoe_ffn_workspace_bytes, 64 MB): one buffer
+    per device and stream, allocated on first use -- kernels of one stream run one after the other, so they can share it."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(_lib.load().picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
 def _down(act, counts, down_w, row_weight):
     lib = _lib.load()
     E, H, I = down_w.shape
     N = act.shape[0]
     y = torch.empty((N, H), dtype=act.dtype, device=act.device)
+    ws = _ffn_workspace(act.device) if act.dtype == torch.bfloat16 else None
     _lib.check(
         lib.picomoe_ffn_down(_lib.ptr(act), _lib.ptr(counts), E, N, H, I, _lib.ptr(down_w), _lib.ptr(row_weight),
-                             _lib.dtype_code(act.dtype), _lib.ptr(y), _lib.stream_ptr()),
+                             _lib.dtype_code(act.dtype), _lib.ptr(y), _lib.ptr(ws), ws.numel() if ws is not None else 0,
+                             _lib.stream_ptr()),
         "picomoe_ffn_down",
     )
     return y
@@ -124,9 +140,11 @@ def _dgrad_x(d13, counts, gate_w, up_w):
     E, I, H = gate_w.shape
     N = d13.shape[0]
     dx = torch.empty((N, H), dtype=d13.dtype, device=d13.device)
+    ws = _ffn_workspace(d13.device) if d13.dtype == torch.bfloat16 else None
     _lib.check(
         lib.picomoe_ffn_dgrad_x(_lib.ptr(d13), _lib.ptr(counts), E, N, H, I, _lib.ptr(gate_w), _lib.ptr(up_w),
-                                _lib.dtype_code(d13.dtype), _lib.ptr(dx), _lib.stream_ptr()),
+                                _lib.dtype_code(d13.dtype), _lib.ptr(dx), _lib.ptr(ws), ws.numel() if ws is not None else 0,
+                                _lib.stream_ptr()),
         "picomoe_ffn_dgrad_x",
     )
     return dx

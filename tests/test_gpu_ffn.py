@@ -123,6 +123,51 @@ def test_bf16_ragged_against_oracle(gpu, H, I, counts):
         assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
 
 
+@pytest.mark.parametrize("counts", [[300, 260, 100, 515], [256, 512, 7, 129], [40, 0, 3, 1]])
+def test_split_last_round_matches_whole_tiles(gpu, counts):
+    """With a workspace the down and dgrad_x kernels cut the tiles of the last, partly filled round into 2 or 4 ranges of K
+    (K here is 32 and 64 k-tiles, enough for 2 and 4 pieces) and add the fp32 partial tiles up in a second kernel: the
+    result must agree with the whole-tile kernels to the rounding of the partial sums, and with the oracle at the bf16
+    tolerance; rows past the tiles' segments must stay untouched."""
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel import megakernel as mk
+
+    E, H, I = len(counts), 512, 2048
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.bfloat16, 11, scale=0.03)
+    N = x.shape[0]
+    act = (torch.randn(N, I, generator=g) * 0.5).bfloat16().cuda()
+    rw = torch.rand(N, generator=g).bfloat16().cuda()
+    d13 = (torch.randn(N, 2 * I, generator=g) * 0.5).bfloat16().cuda()
+    cntd, gwd, uwd, dwd = cnt.cuda(), gw.cuda(), uw.cuda(), dw.cuda()
+    lib = _lib.load()
+    ws = torch.empty(lib.picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device="cuda")
+
+    def down(workspace):
+        y = torch.full((N, H), 7.0, dtype=torch.bfloat16, device="cuda")
+        _lib.check(lib.picomoe_ffn_down(_lib.ptr(act), _lib.ptr(cntd), E, N, H, I, _lib.ptr(dwd), _lib.ptr(rw), _lib.dtype_code(act.dtype),
+                                        _lib.ptr(y), _lib.ptr(workspace), workspace.numel() if workspace is not None else 0,
+                                        _lib.stream_ptr()), "picomoe_ffn_down")
+        return y
+
+    def dgrad_x(workspace):
+        dx = torch.full((N, H), 7.0, dtype=torch.bfloat16, device="cuda")
+        _lib.check(lib.picomoe_ffn_dgrad_x(_lib.ptr(d13), _lib.ptr(cntd), E, N, H, I, _lib.ptr(gwd), _lib.ptr(uwd),
+                                           _lib.dtype_code(d13.dtype), _lib.ptr(dx), _lib.ptr(workspace),
+                                           workspace.numel() if workspace is not None else 0, _lib.stream_ptr()), "picomoe_ffn_dgrad_x")
+        return dx
+
+    owner = torch.repeat_interleave(torch.arange(E), cnt)
+    want_y = torch.einsum("ni,nhi->nh", act.cpu().float(), dw.float()[owner]).bfloat16().float() * rw.cpu().float()[:, None]
+    want_dx = torch.einsum("ni,nih->nh", d13.cpu().float()[:, :I], gw.float()[owner]) + torch.einsum(
+        "ni,nih->nh", d13.cpu().float()[:, I:], uw.float()[owner])
+    for fn, want in ((down, want_y), (dgrad_x, want_dx)):
+        whole, split = fn(None).float().cpu(), fn(ws).float().cpu()
+        scale = want.abs().max()
+        assert (whole - want).abs().max() <= 1e-2 * scale and (split - want).abs().max() <= 1e-2 * scale
+        assert (split - whole).abs().max() <= 2.0 ** -7 * scale       # one bf16 ulp of the largest value
+        assert torch.equal(fn(ws).float().cpu(), split)               # fixed summation order: run to run identical
+
+
 def test_bf16_many_experts(gpu):
     """150 experts (more than one wave's worth in the tile lookup), counts 0..300 incl. empty experts, full tiles and
     tails of both classes: forward and gradients against the oracle."""
