@@ -40,33 +40,51 @@ __global__ __launch_bounds__(kPlanBlock) void plan_hist_kernel(const int64_t* __
 
 // block_hist[b][e] becomes the number of rows of expert e in blocks before b; then experts are laid
 // out back to back using the kept (capacity-limited) counts.
-__global__ __launch_bounds__(256) void plan_scan_kernel(int* __restrict__ block_hist, int n_blocks, int E, int64_t capacity,
-                                                        int64_t slot_lo, int64_t* __restrict__ counts,
-                                                        int64_t* __restrict__ kept_counts, int* __restrict__ seg_start) {
+// One wave per expert (16 waves take the experts in turn): the per-block counts of an expert are scanned 64 blocks at a
+// time with wave shuffles instead of one thread walking all blocks (25 us for 96 blocks x 64 experts, now a few).
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void plan_scan_kernel(int* __restrict__ block_hist, int n_blocks, int E, int64_t capacity,
+                                                                 int64_t slot_lo, int64_t* __restrict__ counts,
+                                                                 int64_t* __restrict__ kept_counts, int* __restrict__ seg_start) {
     __shared__ int kept[kMaxExperts];
-    for (int e = threadIdx.x; e < E; e += 256) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n_waves = kScanThreads / 64;
+    auto wave_scan = [&](int v) {  // inclusive prefix sum over the 64 lanes
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int o = __shfl_up(v, off, 64);
+            if (lane >= off) v += o;
+        }
+        return v;
+    };
+    for (int e = wave; e < E; e += n_waves) {
         int run = 0;
-        for (int b = 0; b < n_blocks; ++b) {
-            const int c = block_hist[(int64_t)b * E + e];
-            block_hist[(int64_t)b * E + e] = run;
-            run += c;
+        for (int b0 = 0; b0 < n_blocks; b0 += 64) {
+            const int b = b0 + lane;
+            const int c = b < n_blocks ? block_hist[(int64_t)b * E + e] : 0;
+            const int incl = wave_scan(c);
+            if (b < n_blocks) block_hist[(int64_t)b * E + e] = run + incl - c;
+            run += __shfl(incl, 63, 64);
         }
-        int64_t kc64 = run;  // rows of e whose rank falls in [slot_lo, slot_lo + capacity)
-        if (capacity > 0) {
-            kc64 = run - slot_lo;
-            kc64 = kc64 < 0 ? 0 : (kc64 > capacity ? capacity : kc64);
+        if (lane == 0) {
+            int64_t kc64 = run;  // rows of e whose rank falls in [slot_lo, slot_lo + capacity)
+            if (capacity > 0) {
+                kc64 = run - slot_lo;
+                kc64 = kc64 < 0 ? 0 : (kc64 > capacity ? capacity : kc64);
+            }
+            kept[e] = (int)kc64;
+            counts[e] = run;
+            kept_counts[e] = kc64;
         }
-        const int kc = (int)kc64;
-        kept[e] = kc;
-        counts[e] = run;
-        kept_counts[e] = kc;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (wave == 0) {  // experts laid out back to back by their kept counts
         int run = 0;
-        for (int e = 0; e < E; ++e) {
-            seg_start[e] = run;
-            run += kept[e];
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int k = e < E ? kept[e] : 0;
+            const int incl = wave_scan(k);
+            if (e < E) seg_start[e] = run + incl - k;
+            run += __shfl(incl, 63, 64);
         }
     }
 }
@@ -329,7 +347,7 @@ extern "C" int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, i
                            block_hist, order);
     }
     const int64_t slot_lo = capacity > 0 ? round_index * capacity : 0;
-    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(256), 0, st, block_hist, n_blocks, E, capacity, slot_lo, counts,
+    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, block_hist, n_blocks, E, capacity, slot_lo, counts,
                        kept_counts, seg_start);
     if (n_rows > 0) {
         int n_bits = 0;
