@@ -5,6 +5,8 @@ import os
 import re
 import types
 
+import ctypes
+
 import pytest
 import torch
 
@@ -40,6 +42,13 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.picomoe_permute_workspace_bytes(1000, 8) > 0
     assert lib.picomoe_permute_workspace_bytes(1000, 5000) == -1
     assert lib.picomoe_route_partials(8192, 8) >= 1
+    # scratch of the split last round: 8 XCDs x 32 partial tiles of 256 x 256 fp32; empty inputs return before any launch
+    assert lib.picomoe_ffn_workspace_bytes() == 8 * 32 * 256 * 256 * 4
+    counts = ctypes.c_void_p(64)   # never dereferenced on the host: these calls return before any launch
+    assert lib.picomoe_ffn_down(null, counts, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 0
+    assert lib.picomoe_ffn_dgrad_x(null, counts, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 0
+    assert lib.picomoe_ffn_down(null, counts, 4, 8, 256, 128, null, null, 1, null, null, 0, null) == 1    # null tensors
+    assert lib.picomoe_ffn_down(null, null, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 1      # null counts
     with pytest.raises(_lib.PicomoeError):
         _lib.check(1, "demo")
 
