@@ -87,21 +87,24 @@ struct GroupedLayout {
     int64_t heavy, light, heavy_per_xcd, light_per_xcd, per_xcd;
     int64_t full;  // slots of whole tiles that come first
     int rem, pieces;
+    int c0;        // this lane's counts[lane] (0 past E): the lookup that follows reuses it instead of loading it again
 };
 
 // Runs in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[] per pass instead of a chain
 // of dependent scalar loads.  Tile and row totals fit 32 bits.
 __device__ __forceinline__ GroupedLayout grouped_layout(const int64_t* counts, int E, int n_tiles, int max_pieces) {
     const int lane = threadIdx.x & 63;
-    int heavy_m = 0, light_m = 0;
+    int heavy_m = 0, light_m = 0, c0 = 0;
     for (int base = 0; base < E; base += 64) {
         const int c = base + lane < E ? (int)counts[base + lane] : 0, rem = c % BM;
+        if (base == 0) c0 = c;
         heavy_m += c / BM + (rem > BM / 2);
         light_m += (rem > 0 && rem <= BM / 2);
     }
     heavy_m = uniform_i32(wave_sum_i32(heavy_m));  // the same in every lane: scalar from here on
     light_m = uniform_i32(wave_sum_i32(light_m));
     GroupedLayout g;
+    g.c0 = c0;
     g.heavy = (int64_t)heavy_m * n_tiles;
     g.light = (int64_t)light_m * n_tiles;
     g.heavy_per_xcd = (g.heavy + kNumXcd - 1) / kNumXcd;
@@ -143,7 +146,7 @@ __device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, i
     }
     int64_t tiles_before = 0, rows_before = 0;
     for (int base = 0; base < E; base += 64) {
-        const int c = base + lane < E ? (int)counts[base + lane] : 0, full = c / BM, rem = c % BM;
+        const int c = base == 0 ? g.c0 : (base + lane < E ? (int)counts[base + lane] : 0), full = c / BM, rem = c % BM;
         const int me = want_light ? (int)(rem > 0 && rem <= BM / 2) : full + (rem > BM / 2);
         const int te = me * n_tiles;
         const int te_incl = wave_scan_i32(te, lane), rows_incl = wave_scan_i32(c, lane);
