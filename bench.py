@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the single-GPU MoE hot path on MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c4|train_step]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c4|c2|train_step]
 
 A "step" is one pass of the hot path over one batch of synthetic input.  The default workload is the
 Mixtral-shape MoE layer forward + backward with FP8 dispatch (8192 tokens, hidden 4096, FFN 14336, 8 experts,
@@ -11,6 +11,9 @@ Inputs and weights are resident in HBM before the clock starts.
 
 `--workload train_step` instead times a whole optimizer step (forward, cross entropy + aux, backward, AdamW) of a
 4-layer Llama whose feed-forward blocks are this MoE layer, the set-up of the reference's tests/bench_ep_train_step.py.
+
+`--workload c2` times the FP8 quantise / dequantise round trip of a 16384 x 4096 bf16 activation on its own, with an
+HBM `roofline` for the quantise kernel and the scalar C oracle as `cpu_baseline`.
 
 Prints ONE JSON line on stdout: the layer's tokens/s as `value`, a `roofline` object for the grouped-GEMM
 kernels (algorithmic FLOP / launch durations measured here with events on the launch stream), the FP8
@@ -31,7 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # L2 <-> memory bytes of the grouped-GEMM launches of one layer step, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE x 2 KiB, WRITE_SIZE x 1 KiB; factors from the --traffic-probe copy kernel).  Algorithmic: 15.5e9.
-MEASURED_TRAFFIC_BYTES = {"c5": 35.2e9}
+MEASURED_TRAFFIC_BYTES = {"c5": 35.2e9, "c2": 201.6e6}  # c2: the quantise kernel alone (algorithmic 201.4e6)
 
 WORKLOADS = {
     # name: tokens, hidden, ffn, experts, top_k, shared, capacity_factor, fp8_dispatch, backward
@@ -281,6 +284,105 @@ def cpu_baseline(w, moe, budget_s=25.0):
     }
 
 
+def traffic_probe(device):
+    """A plain copy kernel of known size (1 GiB read + 1 GiB written per launch, three launches): the reference that
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled by."""
+    import torch
+
+    src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        torch.neg(src, out=dst)
+    torch.cuda.synchronize()
+
+
+def fp8_bench(args):
+    """FP8 E4M3 per-token quantise / dequantise of a 16384 x 4096 bf16 activation (0.1 % outliers of 50 sigma), the
+    dispatch wire format of the reference (picotron/expert_parallel/ep_communications.py:63-68, :100).  A step is one
+    quantise and one dequantise pass over one of six buffer sets (rotated, so every pass comes from HBM and not from
+    the 256 MB last-level cache)."""
+    import numpy as np
+    import torch
+
+    from picotron_amd import _lib
+
+    lib = _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device = torch.device("cuda:0")
+    n, h, sets = 16384, 4096, 6
+    g = torch.Generator(device=device).manual_seed(0)
+    xs = []
+    for _ in range(sets):
+        x = torch.randn(n, h, generator=g, device=device)
+        mask = torch.rand(n, h, generator=g, device=device) < 0.001
+        xs.append(torch.where(mask, 50.0 * torch.randn(n, h, generator=g, device=device), x).bfloat16())
+        del x, mask
+    qs = [torch.empty(n, h, dtype=torch.uint8, device=device) for _ in range(sets)]
+    ss = [torch.empty(n, dtype=torch.float32, device=device) for _ in range(sets)]
+    ys = [torch.empty(n, h, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    st = _lib.stream_ptr()
+    state = {"i": 0}
+
+    def quant():
+        i = state["i"] = (state["i"] + 1) % sets
+        _lib.check(lib.picomoe_fp8_quant(_lib.ptr(xs[i]), 1, n, h, _lib.ptr(qs[i]), _lib.ptr(ss[i]), st), "fp8 quantise")
+
+    def dequant():
+        i = state["i"]
+        _lib.check(lib.picomoe_fp8_dequant(_lib.ptr(qs[i]), _lib.ptr(ss[i]), n, h, _lib.ptr(ys[i]), 1, st), "fp8 dequantise")
+
+    def step():
+        quant()
+        dequant()
+
+    for _ in range(max(args.warmup, sets)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    pass_bytes = n * h * 3 + n * 4
+    # launch durations of each kernel on its own: back-to-back launches between two events on the launch stream
+    tq = time_events(quant, 60, warm=sets)
+    td = time_events(dequant, 60, warm=sets)
+    if args.traffic_probe:
+        traffic_probe(device)
+    rel = float(((ys[0].float() - xs[0].float()).norm() / xs[0].float().norm()).item())
+    log(f"[bench] c2: {ms * 1e3:.1f} us per quantise+dequantise step; quantise {tq * 1e3:.1f} us = "
+        f"{pass_bytes / tq / 1e6:.0f} GB/s, dequantise {td * 1e3:.1f} us = {pass_bytes / td / 1e6:.0f} GB/s, round-trip rel-L2 {rel:.4f}")
+    result = {
+        "metric": "FP8 quant GB/s (per-token E4M3 quantise + dequantise round trip, algorithmic bytes)",
+        "value": 2 * pass_bytes / ms / 1e6, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "FP8 round trip: 16384 x 4096 bf16 -> e4m3 + fp32 row scale -> bf16, 0.1 % outliers",
+                   "rows": n, "hidden": h, "bytes_per_pass": pass_bytes, "round_trip_rel_l2": rel},
+        "roofline": {"bound": "hbm", "achieved": pass_bytes / tq / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": pass_bytes / tq / 1e6 / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
+                     "kernel": "quant_bf16_wave_per_row", "us": tq * 1e3,
+                     "dequant": {"kernel": "dequant_bf16_vec", "achieved": pass_bytes / td / 1e6,
+                                 "frac": pass_bytes / td / 1e6 / HBM_PEAK_GBPS, "us": td * 1e3}},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import c_oracle
+
+        cores = 1
+        rows = 4096  # a quarter of the batch: the scalar C port needs about a second for it
+        bits = xs[0][:rows].cpu().view(torch.int16).numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        q, scale = c_oracle.quant_rows_bf16(bits)
+        c_oracle.dequant_rows_bf16(q, scale)
+        t = time.perf_counter() - t0
+        same = bool((torch.from_numpy(q) == qs[0][:rows].cpu()).all())  # every set was quantised in the timed loop
+        result["cpu_baseline"] = {
+            "value": 2 * (rows * h * 3 + rows * 4) / t / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{rows} of {n} rows, one quantise + dequantise pass of the scalar C oracle in {t:.2f} s",
+        }
+        result["cpu_baseline"]["bytes_equal_gpu"] = same
+    print(json.dumps(result), flush=True)
+
+
 def train_step_bench(args):
     """One optimizer step of a small Llama with MoE feed-forward blocks, the recipe and default sizes of the
     reference's tests/bench_ep_train_step.py:27-44, 54-60, 82-93 (hidden 2048, FFN 2048, 4 layers, 16 heads / 4 kv
@@ -343,7 +445,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + ["train_step"])
+    ap.add_argument("--workload", default="c5", choices=sorted(WORKLOADS) + ["c2", "train_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-times", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -354,6 +456,8 @@ def main():
         sys.exit("bench.py: this build targets one GPU (the EP=1 MoE hot path); run with --gpus 1")
     if args.workload == "train_step":
         return train_step_bench(args)
+    if args.workload == "c2":
+        return fp8_bench(args)
 
     import torch
 
@@ -404,12 +508,7 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     timer.enabled = False
     if args.traffic_probe:
-        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)  # 1 GiB read + 1 GiB written per launch
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.neg(src, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
+        traffic_probe(device)
     tokens_per_s = w["T"] / (ms_per_step * 1e-3)
     log(f"[bench] {args.workload}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tokens/s")
 
