@@ -40,6 +40,15 @@ constexpr int kWaves = PICOMOE_MFMA_WAVES;
 #define PICOMOE_PREFETCH_BWD 2
 #endif
 
+// k-steps per trip of the k-loop, and the modes (bit = Mode) it applies to.  The loop's back edge sits in front of a
+// memory phase, whose fragment reads then start late and hold up the other group's MFMAs: four k-steps per trip gained
+// 1.3 % on the forward and dgrad kernels; wgrad (the most scalar state, which then spills) gained nothing and stays at one.
+#ifndef PICOMOE_KT_UNROLL
+#define PICOMOE_KT_UNROLL 4
+#endif
+#ifndef PICOMOE_KT_UNROLL_MODES
+#define PICOMOE_KT_UNROLL_MODES 0x0F
+#endif
 #ifndef PICOMOE_ROW_BLOCK_SKIP
 #define PICOMOE_ROW_BLOCK_SKIP 1
 #endif
@@ -311,22 +320,25 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage.  The loads are the
     // opaque form: every wait between a load and the LDS reads of its data is written out in this kernel (prologue,
     // sub-step 3 of the k-loop, the end of the loop), the compiler adds none.
-    auto issue_a = [&](int kt, int stage, int q) {
+    // ab / bb: the wave-uniform address of the operand's k-tile; last: it is the segment's last k-tile (wgrad's clamped offsets)
+    auto a_tile = [&](int kt) { return a_base + (int64_t)kt * a_step; };
+    auto b_tile = [&](int kt) { return b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0); };
+    auto issue_a_at = [&](const char* ab, bool last, int stage, int q) {
         char* base = lds + stage * kStageBytes;
-        const char* ab = a_base + (int64_t)kt * a_step;
         if (T::kAKMajor)
             load16_to_lds_opaque(ab, a_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds_opaque(ab, MODE == kWgrad && kt == n_kt - 1 ? a_off_tail[q] : a_off[q], base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(ab, MODE == kWgrad && last ? a_off_tail[q] : a_off[q], base + (wave * KPW + q * 2) * 512);
     };
-    auto issue_b = [&](int kt, int stage, int q) {
+    auto issue_b_at = [&](const char* bb, bool last, int stage, int q) {
         char* base = lds + stage * kStageBytes + kTileBytes;
-        const char* bb = b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0);
         if (T::kBKMajor)
             load16_to_lds_opaque(bb, b_off[q], base + (wave * RPW + q * 8) * 128);
         else
-            load16_to_lds_opaque(bb, MODE == kWgrad && kt == n_kt - 1 ? b_off_tail[q] : b_off[q], base + (wave * KPW + q * 2) * 512);
+            load16_to_lds_opaque(bb, MODE == kWgrad && last ? b_off_tail[q] : b_off[q], base + (wave * KPW + q * 2) * 512);
     };
+    auto issue_a = [&](int kt, int stage, int q) { issue_a_at(a_tile(kt), kt == n_kt - 1, stage, q); };
+    auto issue_b = [&](int kt, int stage, int q) { issue_b_at(b_tile(kt), kt == n_kt - 1, stage, q); };
     auto issue_tile = [&](int kt, int stage) {
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
@@ -476,10 +488,19 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             __builtin_amdgcn_sched_barrier(0);
         };
         if (wm == 1) phase_end();  // the phase offset of the second group
-        for (int kt = 0; kt < n_kt; ++kt) {
+        // The k-tile the loads of a k-step fetch: kt + 1, or the last one again once kt + 1 runs past it (its stage was
+        // last read one k-step ago).  Its operand addresses move on by one k-tile per k-step with two scalar adds;
+        // working them out from kt (64-bit scalar multiplies by the run-time row pitch of an X-major operand) put some
+        // twenty dependent scalar instructions in front of the first load of sub-step 0, between two MFMAs.
+        const int kt_first_next = n_kt > 1 ? 1 : 0;
+        // (readfirstlane: the loads take their base from scalar registers, and the compiler is free to evaluate even
+        // wave-uniform selects like the one in b_tile on the vector unit)
+        const char* a_next = (const char*)uniform_i64((int64_t)(uintptr_t)a_tile(kt_first_next));
+        const char* b_next = (const char*)uniform_i64((int64_t)(uintptr_t)b_tile(kt_first_next));
+        bool next_is_last = kt_first_next == n_kt - 1;
+        auto k_step = [&](int kt) {
             const int stage = kt & 1;
             const bool tail = MODE == kWgrad && kt == n_kt - 1;
-            const int kt_next = kt + 1 < n_kt ? kt + 1 : n_kt - 1;  // its stage was last read one k-step ago
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 // memory phase
@@ -496,15 +517,29 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 mma_with(active, [&](int n) {
                     if (kk < 2 && (n & 1) == 0) {
                         const int q = (QN / 2) * kk + (n >> 2);  // n = 0, 2: loads q of A and B; n = 4, 6: loads q + 1
-                        if ((n & 2) == 0) issue_a(kt_next, stage ^ 1, q);
-                        else issue_b(kt_next, stage ^ 1, q);
+                        if ((n & 2) == 0) issue_a_at(a_next, next_is_last, stage ^ 1, q);
+                        else issue_b_at(b_next, next_is_last, stage ^ 1, q);
                     }
                     if (kk == 2 && n == 1) prefetch_l2(kt);
                 });
-                if (kk == 3) flip_stage();
+                if (kk == 3) {
+                    flip_stage();
+                    if (kt + 2 < n_kt) {  // the next k-step fetches k-tile kt + 2
+                        a_next += a_step;
+                        b_next += b_step + (kt + 2 == b_switch_kt ? b_switch_delta : 0);
+                    }
+                    next_is_last = kt + 2 >= n_kt - 1;
+                }
                 phase_end();
             }
+        };
+        constexpr int kUnroll = ((PICOMOE_KT_UNROLL_MODES >> MODE) & 1) ? PICOMOE_KT_UNROLL : 1;
+        int kt_done = 0;
+        for (; kt_done + kUnroll <= n_kt; kt_done += kUnroll) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) k_step(kt_done + u);
         }
+        for (; kt_done < n_kt; ++kt_done) k_step(kt_done);
         if (wm == 0) phase_end();  // the first group finishes one phase early
     };
     // Five copies of the loop, picked per wave by the number of its 32-row blocks that hold rows of the segment: a wave
