@@ -250,12 +250,20 @@ class _FusedMoE(torch.autograd.Function):
             y0 = _down(act, counts, dw, None)
             d_rw = (dy.float() * y0.float()).sum(dim=1).to(rw.dtype)
             dy = dy * rw[:, None]
-        d13, _ = _dgrad_act(dy, counts, dw, inter13, want_act=False)
-        dx = _dgrad_x(d13, counts, gw, uw)
+        # only the GEMMs whose results autograd asked for (frozen experts, or an input that needs no gradient, skip theirs)
+        want_dx, want_gate, want_up, want_down = ctx.needs_input_grad[:4]
         E, N, H, I = counts.numel(), x.shape[0], x.shape[1], act.shape[1]
-        d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device)
-        d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
-        d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
+        dx = d_gate = d_up = d_down = None
+        if want_dx or want_gate or want_up:
+            d13, _ = _dgrad_act(dy, counts, dw, inter13, want_act=False)
+            if want_dx:
+                dx = _dgrad_x(d13, counts, gw, uw)
+        if want_down:
+            d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device)
+        if want_gate:
+            d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
+        if want_up:
+            d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
         return dx, d_gate, d_up, d_down, None, d_rw, None
 
 

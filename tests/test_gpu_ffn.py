@@ -61,6 +61,25 @@ def test_row_weight_epilogue(gpu):
         assert torch.allclose(a.grad.cpu(), b.grad, atol=1e-4, rtol=1e-4)
 
 
+def test_backward_computes_only_what_autograd_asks_for(gpu):
+    """Frozen experts (input gradient only), and a frozen input with one trainable matrix: the gradients that are asked
+    for equal the oracle's, the others stay None."""
+    from picotron_amd.expert_parallel import megakernel
+
+    x, counts, gw, uw, dw, g = _mk(3, 32, 64, [9, 0, 40], torch.float32, 5)
+    dy = torch.randn(49, 32, generator=g)
+    ref = O.expert_ffn_backward(x, counts, gw, uw, dw, dy)
+    xg = x.cuda().requires_grad_(True)
+    megakernel.fused_moe(xg, counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda()).backward(dy.cuda())
+    assert torch.allclose(xg.grad.cpu(), ref[0], atol=1e-4, rtol=1e-4)
+    for which in (1, 2, 3):
+        leaves = [t.cuda() for t in (x, gw, uw, dw)]
+        leaves[which].requires_grad_(True)
+        megakernel.fused_moe(leaves[0], counts.cuda(), *leaves[1:]).backward(dy.cuda())
+        assert torch.allclose(leaves[which].grad.cpu(), ref[which], atol=1e-4, rtol=1e-4)
+        assert all(l.grad is None for i, l in enumerate(leaves) if i != which)
+
+
 def test_bf16_small(gpu):
     from picotron_amd.expert_parallel import megakernel
 
