@@ -361,7 +361,7 @@ def fp8_bench(args):
         "roofline": {"bound": "hbm", "achieved": pass_bytes / tq / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": pass_bytes / tq / 1e6 / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
                      "kernel": "quant_bf16_wave_per_row", "us": tq * 1e3,
-                     "dequant": {"kernel": "dequant_bf16_vec", "achieved": pass_bytes / td / 1e6,
+                     "dequant": {"kernel": "dequant_bf16_wave_per_row", "achieved": pass_bytes / td / 1e6,
                                  "frac": pass_bytes / td / 1e6 / HBM_PEAK_GBPS, "us": td * 1e3}},
     }
     if not args.no_cpu_baseline:
