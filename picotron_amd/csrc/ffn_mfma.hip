@@ -498,9 +498,12 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         const char* a_next = (const char*)uniform_i64((int64_t)(uintptr_t)a_tile(kt_first_next));
         const char* b_next = (const char*)uniform_i64((int64_t)(uintptr_t)b_tile(kt_first_next));
         bool next_is_last = kt_first_next == n_kt - 1;
-        auto k_step = [&](int kt) {
+        // last_k_tile (compile time): wgrad's last k-tile, whose fragments are masked past the expert's last row.  It is a
+        // copy of the k-step of its own, so that the other k-steps carry no test for it (a compare and a taken branch in
+        // every memory phase, on the path the other group's MFMAs wait for).
+        auto k_step = [&](int kt, auto last_k_tile) {
             const int stage = kt & 1;
-            const bool tail = MODE == kWgrad && kt == n_kt - 1;
+            constexpr bool tail = MODE == kWgrad && decltype(last_k_tile)::value;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 // memory phase
@@ -534,12 +537,14 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             }
         };
         constexpr int kUnroll = ((PICOMOE_KT_UNROLL_MODES >> MODE) & 1) ? PICOMOE_KT_UNROLL : 1;
+        const int n_plain = MODE == kWgrad ? n_kt - 1 : n_kt;  // k-steps without the tail mask
         int kt_done = 0;
-        for (; kt_done + kUnroll <= n_kt; kt_done += kUnroll) {
+        for (; kt_done + kUnroll <= n_plain; kt_done += kUnroll) {
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) k_step(kt_done + u);
+            for (int u = 0; u < kUnroll; ++u) k_step(kt_done + u, std::false_type{});
         }
-        for (; kt_done < n_kt; ++kt_done) k_step(kt_done);
+        for (; kt_done < n_plain; ++kt_done) k_step(kt_done, std::false_type{});
+        if (MODE == kWgrad && n_kt > 0) k_step(n_kt - 1, std::true_type{});
         if (wm == 0) phase_end();  // the first group finishes one phase early
     };
     // Five copies of the loop, picked per wave by the number of its 32-row blocks that hold rows of the segment: a wave
