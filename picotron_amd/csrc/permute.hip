@@ -155,8 +155,10 @@ struct Vec;
 template <>
 struct Vec<uint16_t, 8> {
     float v[8];
-    __device__ __forceinline__ void load(const uint16_t* p) {
-        const u32x4_t w = *(const u32x4_t*)p;
+    typedef u32x4_t raw_t;  // what a load leaves in registers before it is widened to fp32
+    static __device__ __forceinline__ raw_t load_raw(const uint16_t* p) { return *(const u32x4_t*)p; }
+    __device__ __forceinline__ void load(const uint16_t* p) { set(load_raw(p)); }
+    __device__ __forceinline__ void set(raw_t w) {
         const uint32_t a[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -176,21 +178,27 @@ struct Vec<uint16_t, 8> {
 template <>
 struct Vec<uint16_t, 1> {
     float v[1];
+    typedef uint16_t raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const uint16_t* p) { return *p; }
+    __device__ __forceinline__ void set(raw_t w) { v[0] = bf16_bits_to_f32(w); }
     __device__ __forceinline__ void load(const uint16_t* p) { v[0] = bf16_bits_to_f32(*p); }
     __device__ __forceinline__ void store(uint16_t* p) const { *p = (uint16_t)f32_to_bf16_bits(v[0]); }
 };
 template <>
 struct Vec<float, 4> {
     float v[4];
-    __device__ __forceinline__ void load(const float* p) {
-        const f32x4_t w = *(const f32x4_t*)p;
-        v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
-    }
+    typedef f32x4_t raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const float* p) { return *(const f32x4_t*)p; }
+    __device__ __forceinline__ void set(raw_t w) { v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w; }
+    __device__ __forceinline__ void load(const float* p) { set(load_raw(p)); }
     __device__ __forceinline__ void store(float* p) const { *(f32x4_t*)p = f32x4_t{v[0], v[1], v[2], v[3]}; }
 };
 template <>
 struct Vec<float, 1> {
     float v[1];
+    typedef float raw_t;
+    static __device__ __forceinline__ raw_t load_raw(const float* p) { return *p; }
+    __device__ __forceinline__ void set(raw_t w) { v[0] = w; }
     __device__ __forceinline__ void load(const float* p) { v[0] = *p; }
     __device__ __forceinline__ void store(float* p) const { *p = v[0]; }
 };
@@ -222,18 +230,23 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ 
 // out[t] = sum_j w[t,j] * y[inv[t*k+j]].  Each product is rounded to T, the sum is carried in fp32
 // and rounded once: what both a reshape-sum over k and a CPU index_add into a zeroed T buffer do.
 // Rows with inv < 0 (dropped) add nothing.  w == nullptr means unit weights without the product rounding.
-template <typename T, int V>
+// KMAX: compile-time bound of k (2, 8 or kMaxTopK).  A wave works on one token, so the row positions are wave-uniform
+// (kept in scalar registers); per column chunk all of the token's rows are loaded first and summed afterwards, so the
+// k loads are in flight together.
+template <typename T, int V, int KMAX>
 __global__ __launch_bounds__(256) void combine_fwd_kernel(const T* __restrict__ y, const int* __restrict__ inv,
                                                           const T* __restrict__ w, int64_t n_tokens, int k, int64_t hidden,
                                                           T* __restrict__ out) {
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tokens) return;
-    int pos[kMaxTopK];
-    float wj[kMaxTopK];
+    int pos[KMAX];
+    float wj[KMAX];
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
+    for (int j = 0; j < KMAX; ++j) {
+        pos[j] = -1;
+        wj[j] = 0.f;
         if (j < k) {
-            pos[j] = inv ? inv[t * k + j] : (int)(t * k + j);
+            pos[j] = __builtin_amdgcn_readfirstlane(inv ? inv[t * k + j] : (int)(t * k + j));
             if (w) {
                 Vec<T, 1> s;
                 s.load(w + t * k + j);
@@ -244,14 +257,18 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(const T* __restrict__ 
         }
     }
     for (int64_t c = (int64_t)(threadIdx.x & 63) * V; c < hidden; c += 64 * V) {
+        typename Vec<T, V>::raw_t raw[KMAX];
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j)
+            if (pos[j] >= 0) raw[j] = Vec<T, V>::load_raw(y + (int64_t)pos[j] * hidden + c);
         Vec<T, V> acc;
 #pragma unroll
         for (int i = 0; i < V; ++i) acc.v[i] = 0.f;
 #pragma unroll
-        for (int j = 0; j < kMaxTopK; ++j) {
-            if (j < k && pos[j] >= 0) {
+        for (int j = 0; j < KMAX; ++j) {
+            if (pos[j] >= 0) {
                 Vec<T, V> x;
-                x.load(y + (int64_t)pos[j] * hidden + c);
+                x.set(raw[j]);
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
                     const float prod = w ? round_to<T>(x.v[i] * wj[j]) : x.v[i];
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(256) void combine_fwd_kernel(const T* __restrict__ 
 }
 
 // d y[inv[t*k+j]] = w[t,j] * d out[t];   d w[t,j] = <d out[t], y[inv[t*k+j]]>
-template <typename T, int V>
+template <typename T, int V, int KMAX>
 __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ d_out, const T* __restrict__ y,
                                                           const int* __restrict__ inv, const T* __restrict__ w,
                                                           int64_t n_tokens, int k, int64_t hidden, T* __restrict__ d_y,
@@ -272,13 +289,15 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tokens) return;
     const int lane = threadIdx.x & 63;
-    int pos[kMaxTopK];
-    float wj[kMaxTopK], dot[kMaxTopK];
+    int pos[KMAX];
+    float wj[KMAX], dot[KMAX];
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
+    for (int j = 0; j < KMAX; ++j) {
         dot[j] = 0.f;
+        pos[j] = -1;
+        wj[j] = 0.f;
         if (j < k) {
-            pos[j] = inv ? inv[t * k + j] : (int)(t * k + j);
+            pos[j] = __builtin_amdgcn_readfirstlane(inv ? inv[t * k + j] : (int)(t * k + j));
             Vec<T, 1> s;
             s.load(w + t * k + j);
             wj[j] = s.v[0];
@@ -287,11 +306,15 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
     for (int64_t c = (int64_t)lane * V; c < hidden; c += 64 * V) {
         Vec<T, V> g;
         g.load(d_out + t * hidden + c);
+        typename Vec<T, V>::raw_t raw[KMAX];
 #pragma unroll
-        for (int j = 0; j < kMaxTopK; ++j) {
-            if (j < k && pos[j] >= 0) {
+        for (int j = 0; j < KMAX; ++j)
+            if (pos[j] >= 0) raw[j] = Vec<T, V>::load_raw(y + (int64_t)pos[j] * hidden + c);
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) {
+            if (pos[j] >= 0) {
                 Vec<T, V> x, o;
-                x.load(y + (int64_t)pos[j] * hidden + c);
+                x.set(raw[j]);
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
                     o.v[i] = g.v[i] * wj[j];
@@ -302,7 +325,7 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
         }
     }
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
+    for (int j = 0; j < KMAX; ++j) {
         if (j < k) {
             const float tot = wave_sum(dot[j]);
             if (lane == 0) {
@@ -386,20 +409,32 @@ void launch_combine_fwd(hipStream_t st, const void* y, const int* inv, const voi
     const dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
     constexpr int V = sizeof(T) == 2 ? 8 : 4;
     const bool vec = can_vec<T>(hidden, y, out);
-    if (vec)
-        hipLaunchKernelGGL((combine_fwd_kernel<T, V>), grid, block, 0, st, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)out);
-    else
-        hipLaunchKernelGGL((combine_fwd_kernel<T, 1>), grid, block, 0, st, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)out);
+#define PICOMOE_LAUNCH_CF(VV, KK) \
+    hipLaunchKernelGGL((combine_fwd_kernel<T, VV, KK>), grid, block, 0, st, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)out)
+    if (vec) {
+        if (k <= 2) PICOMOE_LAUNCH_CF(V, 2);
+        else if (k <= 8) PICOMOE_LAUNCH_CF(V, 8);
+        else PICOMOE_LAUNCH_CF(V, kMaxTopK);
+    } else {
+        PICOMOE_LAUNCH_CF(1, kMaxTopK);
+    }
+#undef PICOMOE_LAUNCH_CF
 }
 template <typename T>
 void launch_combine_bwd(hipStream_t st, const void* d_out, const void* y, const int* inv, const void* w, int64_t n_tokens,
                         int k, int64_t hidden, void* d_y, void* d_w) {
     const dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
     constexpr int V = sizeof(T) == 2 ? 8 : 4;
-    if (can_vec<T>(hidden, d_out, y, d_y))
-        hipLaunchKernelGGL((combine_bwd_kernel<T, V>), grid, block, 0, st, (const T*)d_out, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)d_y, (T*)d_w);
-    else
-        hipLaunchKernelGGL((combine_bwd_kernel<T, 1>), grid, block, 0, st, (const T*)d_out, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)d_y, (T*)d_w);
+#define PICOMOE_LAUNCH_CB(VV, KK) \
+    hipLaunchKernelGGL((combine_bwd_kernel<T, VV, KK>), grid, block, 0, st, (const T*)d_out, (const T*)y, inv, (const T*)w, n_tokens, k, hidden, (T*)d_y, (T*)d_w)
+    if (can_vec<T>(hidden, d_out, y, d_y)) {
+        if (k <= 2) PICOMOE_LAUNCH_CB(V, 2);
+        else if (k <= 8) PICOMOE_LAUNCH_CB(V, 8);
+        else PICOMOE_LAUNCH_CB(V, kMaxTopK);
+    } else {
+        PICOMOE_LAUNCH_CB(1, kMaxTopK);
+    }
+#undef PICOMOE_LAUNCH_CB
 }
 }  // namespace
 
