@@ -139,3 +139,27 @@ def test_permute_combine_backward(gpu, dtype):
     assert torch.allclose(out.detach().cpu().float(), ref.detach().float(), **tol)
     assert torch.allclose(tg.grad.cpu().float(), tr.grad.float(), **tol)
     assert torch.allclose(wg.grad.cpu().float(), wr.grad.float(), **(dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=0.3)))
+
+
+@pytest.mark.parametrize("k", [1, 2, 6, 12])
+def test_combine_every_top_k_width(gpu, k):
+    """Forward and backward of the combine for each compile-time bound of k the kernels are built for (2, 8, 16)."""
+    from picotron_amd import _ops
+
+    T, E, H = 70, 16, 264
+    g = torch.Generator().manual_seed(k)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    w = torch.softmax(torch.randn(T, k, generator=g), -1).bfloat16()
+    y = torch.randn(T * k, H, generator=g).bfloat16()                  # expert outputs in sorted order
+    gout = torch.randn(T, H, generator=g).bfloat16()
+    plan = _ops.permute_plan(idx.reshape(-1).cuda(), E)
+    yg, wg = y.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    out = _ops.unpermute_combine(yg, wg, plan.inv_order, plan.order, T, k)
+    out.backward(gout.cuda())
+    order, inv, _ = O.permute_plan_fast(idx.reshape(-1), E)
+    yr, wr = y.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    want = O.combine_topk(yr[inv], wr.reshape(-1), T, k)
+    want.backward(gout)
+    assert torch.equal(out.detach().cpu(), want.detach())              # same rounding points as the reference ops
+    assert torch.allclose(yg.grad.cpu().float(), yr.grad.float(), rtol=1e-2, atol=1e-2)
+    assert torch.allclose(wg.grad.cpu().float(), wr.grad.float(), rtol=2e-2, atol=0.3)
