@@ -13,12 +13,14 @@ Reference lines each function follows (paths relative to the reference checkout)
   expert_ffn           picotron/expert_parallel/expert_parallel.py:323-329,
                        picotron/expert_parallel/megakernel.py:308-318, picotron/model.py:258
   silu_and_mul_bwd     picotron/expert_parallel/megakernel.py:187-197
+  expert_ffn_backward_explicit  picotron/expert_parallel/megakernel.py:332-357 (fused_moe_dgrad / fused_moe_wgrad)
   combine_topk         picotron/expert_parallel/expert_parallel.py:219-224
   compute_capacity     picotron/expert_parallel/capacity_moe.py:33-41
   slot_assignment      picotron/expert_parallel/capacity_moe.py:44-57
   capped_forward       picotron/expert_parallel/capacity_moe.py:93-160 (drop mode and dropless rounds)
   quant_fp8 / dequant  picotron/expert_parallel/ep_communications.py:59-68, :100
-  moe_forward          picotron/expert_parallel/expert_parallel.py:144-166, 271-309
+  moe_forward          picotron/expert_parallel/expert_parallel.py:144-166, 271-309; the LatentMoE
+                       projections around the routed path: :59-69, :226-228 (_maybe_down), :250-252 (_finalize)
 
 What pins each function (see tests/test_oracle_*.py):
   * route: brute-force per-row Python selection, torch.topk on tie-free rows, weights sum to one.
@@ -27,8 +29,13 @@ What pins each function (see tests/test_oracle_*.py):
   * capacity: the drop-percentage / round tables the reference README holds (tests/golden/).
   * fp8: closed-form 256-entry decode table; software RNE encoder against
     ``Tensor.to(torch.float8_e4m3fn)`` on every interesting fp32 value; oracle/fp8_e4m3.c.
-  * expert_ffn: a per-token brute-force loop; silu_and_mul_bwd: autograd and finite differences.
-  * moe_forward: a per-token brute-force MoE (each token sent through its experts one at a time).
+  * expert_ffn: a per-token brute-force loop; silu_and_mul_bwd: autograd and finite differences;
+    expert_ffn_backward_explicit: autograd over expert_ffn in float64 (the two are the same mathematics).
+  * moe_forward: a per-token brute-force MoE (each token sent through its experts one at a time);
+    latent: equals the plain layer run on ``tokens @ W_down^T`` (same routing) followed by ``@ W_up^T``,
+    two library matmuls, plus the shared expert on the full-width tokens; dropless rounds: equal to the
+    uncapped layer when ``max_rounds`` covers every row, and to the drop mode at capacity
+    ``max_rounds * C`` when it does not (the rounds partition the rows by rank).
 
 Tie rule for top-k (``torch.topk`` leaves the order of equal scores unspecified): higher score
 first; among equal scores the lower expert id first.  The HIP router uses the same rule.
@@ -177,10 +184,52 @@ def expert_ffn_backward(x_sorted, counts, gate_w, up_w, down_w, dy):
         return torch.autograd.grad(y, leaves, dy)
 
 
+def expert_ffn_backward_explicit(x_sorted, counts, gate_w, up_w, down_w, dy):
+    """(dx, d_gate, d_up, d_down) by the reference's explicit dgrad / wgrad formulas (megakernel.py:332-357, what its
+    ``_FusedMoE.backward`` runs on a GPU), spelled with library matmuls and rounding where those kernels round:
+    ``[g|u]`` and ``da = dy @ down_w`` to the tensor dtype, the SwiGLU backward in fp32 arithmetic rounded once
+    (:187-197), ``dx = [dg|du] @ [gate_w; up_w]`` as ONE contraction over 2I rounded once, the weight gradients as
+    contractions over the expert's rows.  Mathematically the same as ``expert_ffn_backward``; in bf16 the autograd
+    form rounds ``da*u``, ``dg``, ``du`` and the two halves of ``dx`` separately."""
+    dxs, dgs, dus, dds, start = [], [], [], [], 0
+    for e, n in enumerate(counts.tolist()):
+        x, d = x_sorted[start : start + n], dy[start : start + n]
+        inter13 = torch.cat([F.linear(x, gate_w[e]), F.linear(x, up_w[e])], dim=1)
+        a = F.silu(inter13[:, : gate_w.shape[1]]) * inter13[:, gate_w.shape[1] :]
+        da = d @ down_w[e]
+        d13 = silu_and_mul_bwd(inter13, da)
+        dxs.append(d13 @ torch.cat([gate_w[e], up_w[e]], dim=0))
+        dds.append(d.t() @ a)
+        dw13 = d13.t() @ x
+        dgs.append(dw13[: gate_w.shape[1]])
+        dus.append(dw13[gate_w.shape[1] :])
+        start += n
+    dx = torch.cat(dxs, dim=0) if dxs else torch.zeros_like(x_sorted)
+    return dx, torch.stack(dgs), torch.stack(dus), torch.stack(dds)
+
+
+class _ExplicitFfn(torch.autograd.Function):
+    """``expert_ffn`` whose backward is ``expert_ffn_backward_explicit`` (the reference's ``_FusedMoE``,
+    megakernel.py:376-400, without a row weight)."""
+
+    @staticmethod
+    def forward(ctx, x_sorted, counts, gate_w, up_w, down_w):
+        ctx.save_for_backward(x_sorted, gate_w, up_w, down_w)
+        ctx.counts = counts
+        return expert_ffn(x_sorted, counts, gate_w, up_w, down_w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x_sorted, gate_w, up_w, down_w = ctx.saved_tensors
+        dx, dg, du, dd = expert_ffn_backward_explicit(x_sorted, ctx.counts, gate_w, up_w, down_w, dy)
+        return dx, None, dg, du, dd
+
+
 def silu_and_mul_bwd(inter13, da):
     """inter13 = [g | u] ([N,2I]); da [N,I] -> [dg | du] in fp32 arithmetic, cast back."""
     inter = da.shape[1]
-    g, u, d = inter13[:, :inter].float(), inter13[:, inter:].float(), da.float()
+    wide = torch.float64 if inter13.dtype == torch.float64 else torch.float32   # fp32 arithmetic, as the reference
+    g, u, d = inter13[:, :inter].to(wide), inter13[:, inter:].to(wide), da.to(wide)
     s = torch.sigmoid(g)
     dg = d * u * s * (1 + g * (1 - s))
     du = d * g * s
@@ -264,13 +313,16 @@ def dequant_fp8(codes, scale, dtype):
 # ------------------------------------------------------------------------------------------------
 class LayerWeights:
     """Plain container: router [E,H] (+ optional bias [E]), experts gate/up [E,I,H], down [E,H,I],
-    optional shared MLP (gate [Is,H], up [Is,H], down [H,Is]), expert_bias [E] for loss-free balancing."""
+    optional shared MLP (gate [Is,H], up [Is,H], down [H,Is]), expert_bias [E] for loss-free balancing,
+    optional LatentMoE projections ``latent = (down [L,H], up [H,L])`` -- the experts then work in width L
+    (gate/up [E,I,L], down [E,L,I]) while the router and the shared expert keep the full width H."""
 
-    def __init__(self, router_w, gate_w, up_w, down_w, router_b=None, shared=None, expert_bias=None):
+    def __init__(self, router_w, gate_w, up_w, down_w, router_b=None, shared=None, expert_bias=None, latent=None):
         self.router_w, self.router_b = router_w, router_b
         self.gate_w, self.up_w, self.down_w = gate_w, up_w, down_w
         self.shared = shared
         self.expert_bias = expert_bias
+        self.latent = latent
 
     def tensors(self):
         ts = [self.router_w, self.gate_w, self.up_w, self.down_w]
@@ -278,12 +330,17 @@ class LayerWeights:
             ts.append(self.router_b)
         if self.shared is not None:
             ts.extend(self.shared)
+        if self.latent is not None:
+            ts.extend(self.latent)
         return ts
 
 
-def run_local_experts(routed, expert_idx, w):
+def run_local_experts(routed, expert_idx, w, ffn_backward="autograd"):
     order, inv, counts = permute_plan_fast(expert_idx, w.gate_w.shape[0])
-    y_sorted = expert_ffn(routed[order], counts, w.gate_w, w.up_w, w.down_w)
+    if ffn_backward == "explicit":
+        y_sorted = _ExplicitFfn.apply(routed[order], counts, w.gate_w, w.up_w, w.down_w)
+    else:
+        y_sorted = expert_ffn(routed[order], counts, w.gate_w, w.up_w, w.down_w)
     return y_sorted[inv], (order, inv, counts)
 
 
@@ -302,6 +359,8 @@ def moe_forward(
     training=False,
     routing=None,
     logits=None,
+    dispatch_dtype=None,
+    ffn_backward="autograd",
 ):
     """Naive (or capacity-capped) EP=1 MoE layer on [T,H] tokens.  Returns (out [T,H], info dict).
 
@@ -309,7 +368,11 @@ def moe_forward(
     ``_moe_naive`` / ``_moe_capped`` that way); ``logits`` substitutes externally computed router
     logits so a GPU run's own logits can be scored with this selection rule.
     With ``fp8_dispatch`` each routed row goes through quant -> dequant just before the expert FFN
-    (what the reference's FP8 all-to-all does to the rows it ships), gradient straight through.
+    (what the reference's FP8 all-to-all does to the rows it ships), gradient straight through;
+    ``dispatch_dtype`` (test aid) quantises the rows as that dtype would -- amax and scale rounded to it -- when the
+    rest of the layer is evaluated in a wider one (an fp32-arithmetic reference for a bf16 layer).
+    ``ffn_backward``: "autograd" differentiates the expert FFN op by op (the reference on a CPU, megakernel.py:321-329),
+    "explicit" uses its dgrad / wgrad formulas (the reference on a GPU, :332-357); uncapped path only.
     """
     T, H = tokens.shape
     E = w.gate_w.shape[0]
@@ -328,10 +391,14 @@ def moe_forward(
     info.update(topk_idx=topk_idx, topk_w=topk_w)
 
     shared_out = mlp(tokens, *w.shared) if w.shared is not None else None
-    routed, expert_idx, weights, token_idx = expand_routed(tokens, topk_idx, topk_w)
+    # LatentMoE: the routed path runs on the down-projected tokens (a bias-free Linear, rounded to the tensor dtype)
+    routed_in = F.linear(tokens, w.latent[0]) if w.latent is not None else tokens
+    D = routed_in.shape[1]
+    routed, expert_idx, weights, token_idx = expand_routed(routed_in, topk_idx, topk_w)
     if fp8_dispatch:
-        codes, scale = quant_fp8(routed.detach())
-        deq = dequant_fp8(codes, scale, routed.dtype)
+        wire = dispatch_dtype or routed.dtype
+        codes, scale = quant_fp8(routed.detach().to(wire))
+        deq = dequant_fp8(codes, scale, wire).to(routed.dtype)
         routed = routed + (deq - routed).detach()  # value of deq, gradient of identity
         info.update(fp8_codes=codes, fp8_scale=scale)
 
@@ -339,7 +406,7 @@ def moe_forward(
         C = compute_capacity(T, top_k, E, capacity_factor)
         within, counts = slot_assignment(expert_idx, E)
         rounds = capacity_rounds(counts, C, capacity_dropless, max_rounds)
-        out = torch.zeros(T, H, dtype=tokens.dtype)
+        out = torch.zeros(T, D, dtype=tokens.dtype)
         keep_any = torch.zeros_like(within, dtype=torch.bool)
         for r in range(rounds):
             slot = within - r * C
@@ -348,16 +415,18 @@ def moe_forward(
                 continue
             keep_any |= keep
             target = expert_idx[keep] * C + slot[keep]
-            buf = torch.zeros(E * C, H, dtype=tokens.dtype).index_add(0, target, routed[keep])
+            buf = torch.zeros(E * C, D, dtype=tokens.dtype).index_add(0, target, routed[keep])
             ybuf = expert_ffn(buf, torch.full((E,), C, dtype=torch.int64), w.gate_w, w.up_w, w.down_w)
             contrib = ybuf[target] * weights[keep].unsqueeze(-1).to(ybuf.dtype)
-            out = out + torch.zeros(T, H, dtype=tokens.dtype).index_add(0, token_idx[keep], contrib)
+            out = out + torch.zeros(T, D, dtype=tokens.dtype).index_add(0, token_idx[keep], contrib)
         info.update(capacity=C, within=within, counts=counts, keep=keep_any, rounds=rounds)
     else:
-        y, (order, inv, counts) = run_local_experts(routed, expert_idx, w)
+        y, (order, inv, counts) = run_local_experts(routed, expert_idx, w, ffn_backward)
         info.update(order=order, inv_order=inv, counts=counts, y_routed=y)
         out = combine_topk(y, weights, T, top_k)
 
+    if w.latent is not None:  # back up to the full width before the shared expert is added
+        out = F.linear(out, w.latent[1])
     if shared_out is not None:
         out = out + shared_out
     return out, info

@@ -140,10 +140,23 @@ def gather_rows(src, row_map, div, n_out):
     return out
 
 
+def _weights_like(weights, y):
+    """Gate weights in the dtype of the rows they scale: the combine kernels read both as one element type (a bf16
+    weight buffer read as fp32 would be read past its end).  The reference casts the same way
+    (expert_parallel.py:184, capacity_moe.py:158)."""
+    if weights is None:
+        return None
+    if not weights.is_floating_point():
+        raise _lib.PicomoeError(f"combine: gate weights must be floating point, got {weights.dtype}")
+    return weights.to(y.dtype).contiguous()
+
+
 def combine_rows(y, inv_order, weights, n_tokens, top_k):
     lib = _lib.load()
     y = y.contiguous()
-    weights = weights.contiguous() if weights is not None else None
+    weights = _weights_like(weights, y)
+    if weights is not None and weights.numel() != n_tokens * top_k:
+        raise _lib.PicomoeError(f"combine: {weights.numel()} gate weights for {n_tokens} tokens x top-{top_k}")
     out = _empty((n_tokens, y.shape[1]), y.dtype, y.device)
     _lib.check(
         lib.picomoe_combine_fwd(_lib.ptr(y), _lib.ptr(inv_order), _lib.ptr(weights), n_tokens, top_k, y.shape[1],
@@ -181,15 +194,18 @@ class _UnpermuteCombine(torch.autograd.Function):
     @staticmethod
     def forward(ctx, y, weights, inv_order, order, n_tokens, top_k, zero_fill):
         _lib.require_cuda(y)
+        w_dtype = weights.dtype if weights is not None else None
+        y = y.contiguous()
+        weights = _weights_like(weights, y)  # the kernels read weights and rows as one element type
         ctx.save_for_backward(y, weights, inv_order, order)
-        ctx.meta = (n_tokens, top_k, zero_fill)
+        ctx.meta = (n_tokens, top_k, zero_fill, w_dtype)
         return combine_rows(y, inv_order, weights, n_tokens, top_k)
 
     @staticmethod
     def backward(ctx, d_out):
         y, weights, inv_order, order = ctx.saved_tensors
-        n_tokens, top_k, zero_fill = ctx.meta
-        d_out = d_out.contiguous()
+        n_tokens, top_k, zero_fill, w_dtype = ctx.meta
+        d_out = d_out.to(y.dtype).contiguous()
         if weights is None:
             return gather_rows(d_out, order, 1, y.shape[0]), None, None, None, None, None, None
         lib = _lib.load()
@@ -200,7 +216,7 @@ class _UnpermuteCombine(torch.autograd.Function):
                                     y.shape[1], _lib.dtype_code(y.dtype), _lib.ptr(d_y), _lib.ptr(d_w), _lib.stream_ptr()),
             "picomoe_combine_bwd",
         )
-        return d_y, d_w, None, None, None, None, None
+        return d_y, d_w.to(w_dtype), None, None, None, None, None
 
 
 def unpermute_combine(y, weights, inv_order, order, n_tokens, top_k, zero_fill=False):

@@ -170,7 +170,7 @@ class MoELayer(nn.Module):
         if balance and self.use_loss_free:
             with torch.no_grad():
                 self.expert_bias.copy_(bias_f32)
-        return topk_idx, topk_weights
+        return topk_idx, topk_weights.to(tokens.dtype)  # the reference's cast (expert_parallel.py:184)
 
     def _expand_routed(self, tokens, topk_idx, topk_weights):
         """One routed row per (token, selected expert), token-major."""

@@ -139,7 +139,7 @@ def test_bf16_ragged_against_oracle(gpu, H, I, counts):
     y.backward(dy.cuda())
     ref = O.expert_ffn_backward(x.float(), cnt, gw.float(), uw.float(), dw.float(), dy.float())
     for got, want in zip([l.grad for l in leaves], ref):
-        assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
+        assert (got.cpu().float() - want).abs().max() <= 1e-2 * want.abs().max()
 
 
 @pytest.mark.parametrize("counts", [[300, 260, 100, 515], [256, 512, 7, 129], [40, 0, 3, 1]])
@@ -187,6 +187,66 @@ def test_split_last_round_matches_whole_tiles(gpu, counts):
         assert torch.equal(fn(ws).float().cpu(), split)               # fixed summation order: run to run identical
 
 
+@pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32)])
+def test_rows_past_the_segments_are_never_read_into_a_result(gpu, H, I, dtype):
+    """n_rows > sum(counts), as in the capacity modes where the buffers are sized for every routed row and only the kept
+    rows are laid out: the slack rows of every input hold NaN, the slack rows of every output are pre-filled.  Results
+    for the valid rows and all three weight gradients must equal the run without slack bit for bit, and the slack rows
+    of the outputs must come back untouched.  Covers the MFMA kernels (hidden 256) and the generic ones."""
+    from picotron_amd import _lib
+
+    lib = _lib.load()
+    counts = [70, 0, 300, 1, 129]
+    E, n = len(counts), sum(counts)
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, dtype, 13, scale=0.05)
+    dy = torch.randn(n, H, generator=g).to(dtype)
+    cntd, gwd, uwd, dwd = cnt.cuda(), gw.cuda(), uw.cuda(), dw.cuda()
+    code, st = _lib.dtype_code(dtype), _lib.stream_ptr()
+
+    def run(slack):
+        N = n + slack
+        pad = lambda t: torch.cat([t, torch.full((slack, t.shape[1]), float("nan"), dtype=dtype)]).cuda()
+        fill = lambda cols: torch.full((N, cols), 7.0, dtype=dtype, device="cuda")
+        xs, dys = pad(x), pad(dy)
+        act, i13, y, d13, dx = fill(I), fill(2 * I), fill(H), fill(2 * I), fill(H)
+        ws = torch.empty(lib.picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device="cuda")
+        P = _lib.ptr
+        _lib.check(lib.picomoe_ffn_gate_up(P(xs), P(cntd), E, N, H, I, P(gwd), P(uwd), code, P(act), P(i13), st), "gate_up")
+        out_rows = {"act": act.clone(), "inter13": i13.clone()}
+        # slack rows of the intermediates a later kernel reads: NaN, like the caller's torch.empty may hold
+        act[n:], i13[n:] = float("nan"), float("nan")
+        _lib.check(lib.picomoe_ffn_down(P(act), P(cntd), E, N, H, I, P(dwd), None, code, P(y), P(ws), ws.numel(), st), "down")
+        _lib.check(lib.picomoe_ffn_dgrad_act(P(dys), P(cntd), E, N, H, I, P(dwd), P(i13), code, P(d13), None, st), "dgrad_act")
+        out_rows.update(y=y.clone(), d13=d13.clone())
+        d13[n:] = float("nan")
+        _lib.check(lib.picomoe_ffn_dgrad_x(P(d13), P(cntd), E, N, H, I, P(gwd), P(uwd), code, P(dx), P(ws), ws.numel(), st), "dgrad_x")
+        out_rows["dx"] = dx.clone()
+        grads = {}
+        for name, lhs, ld_l, off, rhs, ld_r, p_dim, q_dim in (("d_down", dys, H, 0, act, I, H, I), ("d_gate", d13, 2 * I, 0, xs, H, I, H),
+                                                              ("d_up", d13, 2 * I, I, xs, H, I, H)):
+            o = torch.full((E, p_dim, q_dim), 7.0, dtype=dtype, device="cuda")
+            lp = _lib.ctypes.c_void_p(lhs.data_ptr() + off * lhs.element_size())
+            _lib.check(lib.picomoe_ffn_wgrad(lp, ld_l, P(rhs), ld_r, P(cntd), E, N, p_dim, q_dim, code, P(o), st), name)
+            grads[name] = o
+        torch.cuda.synchronize()
+        return out_rows, grads
+
+    base_rows, base_grads = run(0)
+    rows, grads = run(37)
+    for name, t in rows.items():
+        assert torch.isfinite(t[:n]).all(), name
+        assert torch.equal(t[:n], base_rows[name]), name          # valid rows: bit-identical to the run without slack
+        assert torch.all(t[n:] == 7.0), name                       # slack rows of the outputs: untouched
+    for name, t in grads.items():
+        assert torch.isfinite(t).all(), name
+        assert torch.equal(t, base_grads[name]), name
+        assert torch.all(t[1] == 0), name                          # the empty expert
+    # and the valid rows are the oracle's
+    yr = O.expert_ffn(x, cnt, gw, uw, dw)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert (rows["y"][:n].cpu().float() - yr.float()).abs().max() <= tol * yr.float().abs().max()
+
+
 def test_bf16_many_experts(gpu):
     """150 experts (more than one wave's worth in the tile lookup), counts 0..300 incl. empty experts, full tiles and
     tails of both classes: forward and gradients against the oracle."""
@@ -206,7 +266,7 @@ def test_bf16_many_experts(gpu):
     y.backward(dy.cuda())
     ref = O.expert_ffn_backward(x.float(), cnt, gw.float(), uw.float(), dw.float(), dy.float())
     for got, want in zip([l.grad for l in leaves], ref):
-        assert (got.cpu().float() - want).abs().max() <= 2e-2 * want.abs().max()
+        assert (got.cpu().float() - want).abs().max() <= 1e-2 * want.abs().max()
     assert torch.all(leaves[1].grad[3] == 0) and torch.all(leaves[3].grad[100] == 0)   # empty experts
 
 

@@ -31,7 +31,37 @@ def oracle_weights(moe):
     if moe.shared_expert is not None:
         s = moe.shared_expert
         w.shared = (c(s.gate_proj.weight), c(s.up_proj.weight), c(s.down_proj.weight))
+    if moe.latent:
+        w.latent = (c(moe.down_proj_latent.weight), c(moe.up_proj_latent.weight))
     return w
+
+
+def layer_grads(moe):
+    """The layer's parameter gradients in the order of ``LayerWeights.tensors()``."""
+    gs = [moe.gate.weight.grad] + [torch.stack([getattr(e, n).weight.grad for e in moe.local_experts])
+                                   for n in ("gate_proj", "up_proj", "down_proj")]
+    if moe.gate.bias is not None:
+        gs.append(moe.gate.bias.grad)
+    if moe.shared_expert is not None:
+        gs += [getattr(moe.shared_expert, n).weight.grad for n in ("gate_proj", "up_proj", "down_proj")]
+    if moe.latent:
+        gs += [moe.down_proj_latent.weight.grad, moe.up_proj_latent.weight.grad]
+    return [g.detach().cpu().float() for g in gs]
+
+
+def given_logits(x, w, logits_gpu):
+    """Router logits with the VALUES the GPU computed and the gradient of the oracle's own gate Linear: the GPU's GEMM
+    and the CPU's round a bf16 logit differently now and then, which flips near-tie picks; scoring the GPU's logits
+    with the oracle's selection rule keeps the comparison about the kernels.  a + (b - a) is exact in fp32 for two
+    nearby low-precision values."""
+    own = torch.nn.functional.linear(x, w.router_w, w.router_b)
+    return (own.float() + (logits_gpu.float() - own.float()).detach()).to(own.dtype)
+
+
+def assert_close(got, want, rtol, what=""):
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    err, scale = (got - want).abs().max().item(), want.abs().max().item()
+    assert err <= rtol * scale, f"{what}: max |err| {err:.3e} > {rtol} x {scale:.3e}"
 
 
 def build(cfg, seed=0, std=None, dtype=torch.float32):
@@ -83,9 +113,8 @@ def test_gradients_match_oracle_autograd(gpu, latent):
     out = moe(xg)
     gout = torch.randn(out.shape, generator=torch.Generator().manual_seed(5))
     out.backward(gout.cuda())
-    if latent:
-        return  # the oracle has no latent projections; the dropless == naive test below covers that path
     w = oracle_weights(moe)
+    assert (w.latent is not None) == bool(latent) and w.gate_w.shape[2] == (latent or 32)
     for t in w.tensors():
         t.requires_grad_(True)
     xr = x.view(-1, 32).clone().requires_grad_(True)
@@ -93,13 +122,35 @@ def test_gradients_match_oracle_autograd(gpu, latent):
     ref.backward(gout.view(-1, 32))
     assert torch.allclose(out.detach().cpu().view(-1, 32), ref.detach(), atol=1e-5)
     assert torch.allclose(xg.grad.cpu().view(-1, 32), xr.grad, atol=1e-5)
-    assert torch.allclose(moe.gate.weight.grad.cpu(), w.router_w.grad, atol=1e-5)
-    for i, e in enumerate(moe.local_experts):
-        assert torch.allclose(e.gate_proj.weight.grad.cpu(), w.gate_w.grad[i], atol=1e-5)
-        assert torch.allclose(e.up_proj.weight.grad.cpu(), w.up_w.grad[i], atol=1e-5)
-        assert torch.allclose(e.down_proj.weight.grad.cpu(), w.down_w.grad[i], atol=1e-5)
-    for got, want in zip((moe.shared_expert.gate_proj, moe.shared_expert.up_proj, moe.shared_expert.down_proj), w.shared):
-        assert torch.allclose(got.weight.grad.cpu(), want.grad, atol=1e-5)
+    for got, want in zip(layer_grads(moe), w.tensors()):   # router, experts, shared expert, latent projections
+        assert torch.allclose(got, want.grad, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+def test_latent_layer_matches_oracle(gpu, dtype, rtol):
+    """LatentMoE (reference expert_parallel.py:59-69, 226-228, 250-252) at a size the MFMA kernels tile: hidden 512,
+    latent 256, with the FP8 dispatch on the latent rows in the bf16 case; forward and every gradient."""
+    fp8 = dtype == torch.bfloat16
+    cfg = make_config(hidden=512, inter=256, num_experts=4, top_k=2, n_shared=1, latent=256, ep_fp8_dispatch=fp8)
+    moe = build(cfg, seed=6, std=0.06, dtype=dtype)
+    x = torch.randn(3, 50, 512, generator=torch.Generator().manual_seed(7)).to(dtype)
+    gout = torch.randn(150, 512, generator=torch.Generator().manual_seed(8)).to(dtype)
+    xg = x.cuda().requires_grad_(True)
+    out = moe(xg)
+    out.backward(gout.view_as(out).cuda())
+    w = oracle_weights(moe)
+    for t in w.tensors():
+        t.requires_grad_(True)
+    xr = x.view(-1, 512).clone().requires_grad_(True)
+    logits = given_logits(xr, w, moe.gate(xg.detach().view(-1, 512)).detach().cpu())
+    ref, info = O.moe_forward(xr, w, 2, logits=logits, fp8_dispatch=fp8)
+    ref.backward(gout)
+    assert info["y_routed"].shape[1] == 256
+    assert_close(out.view(-1, 512), ref, rtol, "out")
+    assert_close(xg.grad.view(-1, 512), xr.grad, rtol, "d x")
+    names = ["router", "gate", "up", "down", "shared gate", "shared up", "shared down", "latent down", "latent up"]
+    for name, got, want in zip(names, layer_grads(moe), w.tensors()):
+        assert_close(got, want.grad, rtol, "d " + name)
 
 
 def _run(moe, x):
@@ -132,6 +183,50 @@ def test_capacity_capped_drops_matches_oracle(gpu):
     assert (out_base - out_capped).abs().max().item() > 0
     ref, info = O.moe_forward(x.view(-1, 16), oracle_weights(moe), 2, capacity_factor=0.5, capacity_dropless=False)
     assert torch.allclose(out_capped.cpu(), ref, atol=1e-5)
+
+
+def _zipf_layer(dtype, max_rounds, dropless=True, cap=0.25):
+    """8 experts, top-2, a Zipf bias on the gate so the first experts overflow their capacity several times over."""
+    cfg = make_config(hidden=256, inter=128, num_experts=8, top_k=2, n_shared=1, ep_capacity_factor=cap,
+                      ep_capacity_dropless=dropless, ep_max_rounds=max_rounds)
+    moe = build(cfg, seed=21, std=0.08, dtype=torch.float32)
+    moe.gate.bias = torch.nn.Parameter(-1.5 * torch.log(torch.arange(1, 9, dtype=torch.float32)).cuda())
+    return moe.to(dtype)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("max_rounds", [64, 2])
+def test_dropless_rounds_match_oracle(gpu, dtype, rtol, max_rounds):
+    """Static-memory dropless capacity (reference capacity_moe.py:96-120) under a skewed router that needs at least
+    three rounds: outputs and gradients against the oracle's rounds, with enough rounds (nothing lost) and with
+    ``ep_max_rounds`` = 2, smaller than needed (rows of rank >= 2C are lost, and get no gradient)."""
+    moe = _zipf_layer(dtype, max_rounds)
+    T, H = 384, 256
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(22)).to(dtype)
+    gout = torch.randn(T, H, generator=torch.Generator().manual_seed(23)).to(dtype)
+    xg = x.cuda().requires_grad_(True)
+    out = moe(xg.view(2, T // 2, H))
+    out.backward(gout.view_as(out).cuda())
+    w = oracle_weights(moe)
+    for t in w.tensors():
+        t.requires_grad_(True)
+    xr = x.clone().requires_grad_(True)
+    logits = given_logits(xr, w, moe.gate(xg.detach()).detach().cpu())
+    ref, info = O.moe_forward(xr, w, 2, logits=logits, capacity_factor=0.25, capacity_dropless=True, max_rounds=max_rounds)
+    ref.backward(gout)
+    C = info["capacity"]
+    need = -(-int(info["counts"].max()) // C)
+    assert C == 24 and need >= 3, (C, need)
+    assert info["rounds"] == min(need, max_rounds)
+    assert bool(info["keep"].all()) == (max_rounds >= need)
+    assert_close(out.view(T, H), ref, rtol, "out")
+    assert_close(xg.grad, xr.grad, rtol, "d x")
+    names = ["router", "gate", "up", "down", "router bias", "shared gate", "shared up", "shared down"]
+    for name, got, want in zip(names, layer_grads(moe), w.tensors()):
+        assert_close(got, want.grad, rtol, "d " + name)
+    if max_rounds < need:   # the cut really lost rows: the uncapped layer differs
+        base, _ = O.moe_forward(x, w, 2, logits=logits.detach())
+        assert (base.float() - ref.detach().float()).abs().max() > 10 * rtol * ref.detach().float().abs().max()
 
 
 def test_aux_loss_and_loss_free_bias(gpu):
@@ -195,7 +290,41 @@ def test_fp8_dispatch_bf16(gpu):
     w = oracle_weights(moe)
     ref, info = O.moe_forward(x.view(-1, 256), w, 2, fp8_dispatch=True)
     got = out_fp8.detach().cpu().float().view(-1, 256)
-    assert (got - ref.float()).abs().max() <= 2e-2 * ref.float().abs().max()
+    assert (got - ref.float()).abs().max() <= 1e-2 * ref.float().abs().max()
+
+
+@pytest.mark.parametrize("arith", ["bf16", "fp32"])
+def test_fp8_dispatch_aux_forward_backward_small(gpu, arith):
+    """The headline configuration in small (hidden 256, FFN 512, 8 experts, top-2, bf16, FP8 dispatch, aux-loss
+    coefficient 0.01, training mode, loss = <out, g> + aux): output, aux and every gradient within 1e-2 of the oracle
+    -- once with the oracle in the layer's own bf16 (the reference's rounding points), once with the same weights
+    and inputs evaluated in fp32 arithmetic (the rows still quantised as bf16 rows)."""
+    from picotron_amd.expert_parallel.expert_parallel import collect_aux_loss
+
+    cfg = make_config(hidden=256, inter=512, num_experts=8, top_k=2, ep_fp8_dispatch=True, router_aux_loss_coef=0.01)
+    moe = build(cfg, seed=0, std=0.05, dtype=torch.bfloat16).train()
+    T, H = 1024, 256
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(31)).bfloat16()
+    gout = torch.randn(T, H, generator=torch.Generator().manual_seed(32)).bfloat16()
+    xg = x.cuda().requires_grad_(True)
+    out = moe(xg.view(4, 256, H))
+    aux = collect_aux_loss(moe)
+    torch.autograd.backward([out, aux], [gout.view_as(out).cuda(), torch.ones_like(aux)])
+    wide = torch.float32 if arith == "fp32" else torch.bfloat16
+    w = oracle_weights(moe)
+    w.router_w, w.gate_w, w.up_w, w.down_w = (t.to(wide) for t in (w.router_w, w.gate_w, w.up_w, w.down_w))
+    for t in w.tensors():
+        t.requires_grad_(True)
+    xr = x.to(wide).requires_grad_(True)
+    logits = given_logits(xr, w, moe.gate(xg.detach()).detach().cpu())
+    ref, info = O.moe_forward(xr, w, 2, logits=logits, fp8_dispatch=True, aux_coef=0.01, training=True,
+                              dispatch_dtype=torch.bfloat16)
+    torch.autograd.backward([ref, info["aux"]], [gout.to(wide), torch.ones(())])
+    assert abs(aux.item() - info["aux"].item()) <= 1e-5 * abs(info["aux"].item())
+    assert_close(out.view(T, H), ref, 1e-2, "out")
+    assert_close(xg.grad, xr.grad, 1e-2, "d x")
+    for name, got, want in zip(["router", "gate", "up", "down"], layer_grads(moe), w.tensors()):
+        assert_close(got, want.grad, 1e-2, "d " + name)
 
 
 def test_state_dict_names_and_weight_stacking(gpu):

@@ -138,7 +138,10 @@ def test_permute_combine_backward(gpu, dtype):
     tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
     assert torch.allclose(out.detach().cpu().float(), ref.detach().float(), **tol)
     assert torch.allclose(tg.grad.cpu().float(), tr.grad.float(), **tol)
-    assert torch.allclose(wg.grad.cpu().float(), wr.grad.float(), **(dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=0.3)))
+    if dtype == torch.float32:
+        assert torch.allclose(wg.grad.cpu().float(), wr.grad.float(), rtol=1e-5, atol=1e-5)
+    else:  # bf16 gradients: within 1e-2 of the tensor's magnitude
+        assert (wg.grad.cpu().float() - wr.grad.float()).abs().max() <= 1e-2 * wr.grad.float().abs().max()
 
 
 @pytest.mark.parametrize("k", [1, 2, 6, 12])
@@ -162,4 +165,4 @@ def test_combine_every_top_k_width(gpu, k):
     want.backward(gout)
     assert torch.equal(out.detach().cpu(), want.detach())              # same rounding points as the reference ops
     assert torch.allclose(yg.grad.cpu().float(), yr.grad.float(), rtol=1e-2, atol=1e-2)
-    assert torch.allclose(wg.grad.cpu().float(), wr.grad.float(), rtol=2e-2, atol=0.3)
+    assert (wg.grad.cpu().float() - wr.grad.float()).abs().max() <= 1e-2 * wr.grad.float().abs().max()

@@ -166,6 +166,25 @@ def test_cpu_tensors_are_refused_not_silently_computed():
         assert megakernel.cuda_available() is False
 
 
+def test_combine_weights_follow_the_rows_dtype():
+    """The combine kernels read gate weights and rows as one element type: the wrappers cast the weights to the rows'
+    dtype (as the reference does, expert_parallel.py:184, capacity_moe.py:158) and refuse non-float or mis-sized ones
+    before anything reaches a kernel."""
+    from picotron_amd import _ops
+
+    y = torch.zeros(6, 8, dtype=torch.bfloat16)
+    w = torch.rand(3, 2, dtype=torch.float32)
+    cast = _ops._weights_like(w, y)
+    assert cast.dtype == torch.bfloat16 and cast.is_contiguous() and torch.equal(cast, w.bfloat16())
+    assert _ops._weights_like(None, y) is None
+    assert _ops._weights_like(w.bfloat16().t().contiguous().t(), y.float()).dtype == torch.float32
+    with pytest.raises(_lib.PicomoeError):
+        _ops._weights_like(torch.ones(3, 2, dtype=torch.int64), y)
+    if os.path.exists(_lib.LIB_PATH):
+        with pytest.raises(_lib.PicomoeError):  # 5 weights for 3 tokens x top-2: refused on the host
+            _ops.combine_rows(y, torch.zeros(6, dtype=torch.int32), torch.rand(5), 3, 2)
+
+
 def test_product_does_not_import_the_oracle():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     for dirpath, _, files in os.walk(os.path.join(root, "picotron_amd")):
