@@ -22,12 +22,13 @@ extern "C" {
 
 #define PICOMOE_OK 0
 #define PICOMOE_ERR_ARG 1
+#define PICOMOE_ERR_TOO_LARGE 2
 #define PICOMOE_ERR_HIP_BASE 1000
 
 #define PICOMOE_F32 0
 #define PICOMOE_BF16 1
 
-#define PICOMOE_ABI_VERSION 2
+#define PICOMOE_ABI_VERSION 3
 
 /* ABI version of the loaded library (compare with PICOMOE_ABI_VERSION). */
 int picomoe_abi_version(void);
@@ -87,6 +88,21 @@ int64_t picomoe_permute_workspace_bytes(int64_t n_rows, int num_experts);
 int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
                          int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts, int32_t* within, void* workspace,
                          void* stream);
+
+/* The same plan for callers that cannot allocate or pass a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The block histograms and segment starts
+ * live in a fixed array of PICOMOE_PLAN_STATIC_BYTES (1 MiB) of device memory inside the library, one per GPU, held
+ * until the process ends; the call allocates and frees nothing.  Inputs whose
+ * picomoe_permute_workspace_bytes(n_rows, num_experts) exceeds that -- (ceil(n_rows / 1024) + 1) * num_experts * 4
+ * bytes, e.g. more than 261120 rows at 1024 experts or 33 million rows at 8 -- are refused with PICOMOE_ERR_TOO_LARGE.
+ * Every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU (different streams or threads)
+ * race; calls on one stream are ordered.  Nothing in the array has to be cleared between calls (each call writes every
+ * entry before reading it).  Results are identical to picomoe_permute_plan's. */
+#define PICOMOE_PLAN_STATIC_BYTES (1 << 20)
+int64_t picomoe_permute_plan_static_max_bytes(void);
+int picomoe_permute_plan_static(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
+                                int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts,
+                                int32_t* within, void* stream);
 
 /* Replaces the gathers tokens[token_idx] (EP/expert_parallel.py:216-217) and x[order] (:340) in one pass:
  * out[i] = src[row_map[i] / div] for i < n_out (row_map NULL = identity, negative entries are skipped). */

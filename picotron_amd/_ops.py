@@ -100,7 +100,9 @@ class Plan:
     capacity: int = 0
 
 
-def permute_plan(expert_idx, num_experts, capacity=0, round_index=0, want_within=False):
+def permute_plan(expert_idx, num_experts, capacity=0, round_index=0, want_within=False, static_scratch=False):
+    """``static_scratch``: run the plan on the library's fixed 1 MiB scratch array (``picomoe_permute_plan_static``: no
+    workspace tensor) instead of a workspace allocated here; inputs too large for it are refused."""
     _lib.require_cuda(expert_idx)
     lib = _lib.load()
     expert_idx = expert_idx.contiguous().to(torch.int64)
@@ -114,6 +116,16 @@ def permute_plan(expert_idx, num_experts, capacity=0, round_index=0, want_within
     ws_bytes = lib.picomoe_permute_workspace_bytes(R, num_experts)
     if ws_bytes < 0:
         raise _lib.PicomoeError(f"permute plan: unsupported size (rows={R}, experts={num_experts})")
+    if static_scratch:
+        with torch.cuda.device(dev):  # the library looks its scratch array up on the current device
+            _lib.check(
+                lib.picomoe_permute_plan_static(
+                    _lib.ptr(expert_idx), R, num_experts, int(capacity), int(round_index), _lib.ptr(order), _lib.ptr(inv),
+                    _lib.ptr(counts), _lib.ptr(kept), _lib.ptr(within), _lib.stream_ptr(),
+                ),
+                "picomoe_permute_plan_static",
+            )
+        return Plan(order, inv, counts, kept, within, int(capacity))
     ws = _empty((max(ws_bytes, 4),), torch.uint8, dev)
     _lib.check(
         lib.picomoe_permute_plan(

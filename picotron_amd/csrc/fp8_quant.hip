@@ -294,6 +294,9 @@ extern "C" int picomoe_abi_version(void) { return PICOMOE_ABI_VERSION; }
 extern "C" const char* picomoe_error_string(int code) {
     if (code == PICOMOE_OK) return "ok";
     if (code == PICOMOE_ERR_ARG) return "picomoe: unsupported shape, dtype, alignment or null pointer";
+    if (code == PICOMOE_ERR_TOO_LARGE)
+        return "picomoe: the input is larger than the fixed scratch of this no-allocation entry point "
+               "(use the variant that takes a workspace)";
     if (code >= PICOMOE_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(code - PICOMOE_ERR_HIP_BASE));
     return "picomoe: unknown error code";
 }

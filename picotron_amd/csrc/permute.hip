@@ -8,6 +8,8 @@
 //   combine  out[t] = sum_j w[t,j] * y[inv[t*k+j]]   and its backward
 //
 // All row movers use one wavefront per row and 16-byte lanes when the row width allows it.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -354,18 +356,19 @@ extern "C" int64_t picomoe_permute_workspace_bytes(int64_t n_rows, int num_exper
     return (n_blocks * num_experts + num_experts) * (int64_t)sizeof(int);
 }
 
-extern "C" int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
-                                    int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts,
-                                    int32_t* within, void* workspace, void* stream) {
-    PICOMOE_CHECK_ARG(n_rows >= 0 && n_rows < (1ll << 31) && num_experts >= 1 && num_experts <= kMaxExperts && capacity >= 0 && round_index >= 0);
-    PICOMOE_CHECK_ARG(counts && kept_counts && workspace);
-    hipStream_t st = (hipStream_t)stream;
-    const int E = num_experts;
+// Scratch of the no-allocation entry point (picomoe_permute_plan_static): file scope, one copy per GPU.
+constexpr int64_t kStaticPlanInts = PICOMOE_PLAN_STATIC_BYTES / (int64_t)sizeof(int);
+static __device__ __align__(256) int scratch[kStaticPlanInts];
+
+namespace {
+// the three launches of a plan; `workspace` holds n_blocks * E block histograms followed by E segment starts (ints).
+// Every entry that is read has been written by an earlier launch of the same call: nothing has to start at zero.
+int plan_launch(const int64_t* expert_idx, int64_t n_rows, int E, int64_t capacity, int64_t round_index, int32_t* order,
+                int32_t* inv_order, int64_t* counts, int64_t* kept_counts, int32_t* within, int* workspace, hipStream_t st) {
     const int n_blocks = (int)((n_rows + kPlanChunk - 1) / kPlanChunk);
-    int* block_hist = (int*)workspace;
+    int* block_hist = workspace;
     int* seg_start = block_hist + (int64_t)n_blocks * E;
     if (n_rows > 0) {
-        PICOMOE_CHECK_ARG(expert_idx && order && inv_order);
         hipLaunchKernelGGL(plan_hist_kernel, dim3(n_blocks), dim3(kPlanBlock), E * sizeof(int), st, expert_idx, n_rows, E,
                            block_hist, order);
     }
@@ -379,6 +382,63 @@ extern "C" int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, i
                            E, n_bits, capacity, slot_lo, block_hist, seg_start, order, inv_order, within);
     }
     return picomoe_launch_status();
+}
+
+bool plan_args_ok(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity, int64_t round_index,
+                  const int32_t* order, const int32_t* inv_order, const int64_t* counts, const int64_t* kept_counts) {
+    if (!(n_rows >= 0 && n_rows < (1ll << 31) && num_experts >= 1 && num_experts <= kMaxExperts && capacity >= 0 && round_index >= 0))
+        return false;
+    if (!counts || !kept_counts) return false;
+    return n_rows == 0 || (expert_idx && order && inv_order);
+}
+
+// ---- the plan without a caller-provided workspace -------------------------------------------------------------
+// Scratch of the no-allocation entry point: block histograms + segment starts of one plan, 1 MiB per GPU, held from the
+// moment the library is loaded until the process ends.  In host code `scratch` is only a handle for
+// hipGetSymbolAddress; kernels get the device address that call returns (each GPU has its own copy of the array).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU, looked up on the first call there
+
+// Device address of this GPU's scratch array (looked up once per device, with that device current), or null + *rc.
+int* static_scratch(int* rc) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *rc = PICOMOE_ERR_HIP_BASE + (int)e; return nullptr; }
+    if (dev < 0 || dev >= kMaxDevices) { *rc = PICOMOE_ERR_ARG; return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) { *rc = PICOMOE_ERR_HIP_BASE + (int)(e != hipSuccess ? e : hipErrorInvalidSymbol); return nullptr; }
+        g_scratch_ptr[dev] = (int*)ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
+                                    int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts,
+                                    int32_t* within, void* workspace, void* stream) {
+    PICOMOE_CHECK_ARG(plan_args_ok(expert_idx, n_rows, num_experts, capacity, round_index, order, inv_order, counts, kept_counts));
+    PICOMOE_CHECK_ARG(workspace);
+    return plan_launch(expert_idx, n_rows, num_experts, capacity, round_index, order, inv_order, counts, kept_counts, within,
+                       (int*)workspace, (hipStream_t)stream);
+}
+
+extern "C" int64_t picomoe_permute_plan_static_max_bytes(void) { return PICOMOE_PLAN_STATIC_BYTES; }
+
+extern "C" int picomoe_permute_plan_static(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
+                                           int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts,
+                                           int64_t* kept_counts, int32_t* within, void* stream) {
+    PICOMOE_CHECK_ARG(plan_args_ok(expert_idx, n_rows, num_experts, capacity, round_index, order, inv_order, counts, kept_counts));
+    const int64_t need = picomoe_permute_workspace_bytes(n_rows, num_experts);
+    if (need < 0 || need > PICOMOE_PLAN_STATIC_BYTES) return PICOMOE_ERR_TOO_LARGE;
+    int rc = PICOMOE_OK;
+    int* ws = static_scratch(&rc);
+    if (!ws) return rc;
+    return plan_launch(expert_idx, n_rows, num_experts, capacity, round_index, order, inv_order, counts, kept_counts, within, ws,
+                       (hipStream_t)stream);
 }
 
 extern "C" int picomoe_gather_rows(const void* src, const int32_t* row_map, int div, int64_t n_out, int64_t hidden,
