@@ -29,29 +29,13 @@
 namespace {
 
 constexpr int BK = 64;
-#ifndef PICOMOE_MFMA_WAVES
-#define PICOMOE_MFMA_WAVES 8
-#endif
-constexpr int kWaves = PICOMOE_MFMA_WAVES;
-#ifndef PICOMOE_PREFETCH_FWD
-#define PICOMOE_PREFETCH_FWD 2
-#endif
-#ifndef PICOMOE_PREFETCH_BWD
-#define PICOMOE_PREFETCH_BWD 2
-#endif
-
-// k-steps per trip of the k-loop, and the modes (bit = Mode) it applies to.  The loop's back edge sits in front of a
-// memory phase, whose fragment reads then start late and hold up the other group's MFMAs: four k-steps per trip gained
-// 1.3 % on the forward and dgrad kernels; wgrad (the most scalar state, which then spills) gained nothing and stays at one.
-#ifndef PICOMOE_KT_UNROLL
-#define PICOMOE_KT_UNROLL 4
-#endif
-#ifndef PICOMOE_KT_UNROLL_MODES
-#define PICOMOE_KT_UNROLL_MODES 0x0F
-#endif
-#ifndef PICOMOE_ROW_BLOCK_SKIP
-#define PICOMOE_ROW_BLOCK_SKIP 1
-#endif
+constexpr int kWaves = 8;
+// L2 prefetch distance in k-steps (2 for every mode: 1 cost the backward kernels 9 %, 3 and 4 nothing or 1 %)
+constexpr int kPrefetchDist = 2;
+// k-steps per trip of the k-loop.  The loop's back edge sits in front of a memory phase, whose fragment reads then start
+// late and hold up the other group's MFMAs: four k-steps per trip gained 1.3 % on the forward and dgrad kernels; wgrad
+// (the most scalar state, which then spills) gained nothing and stays at one.
+constexpr int kKtUnroll = 4;
 enum Mode { kGateUp = 0, kDown = 1, kDgradAct = 2, kDgradX = 3, kWgrad = 4 };
 
 template <int MODE>
@@ -88,9 +72,6 @@ __device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >
 
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(8))) short s16x8_t;
-__device__ __forceinline__ s16x4_t lds_read_tr(const char* p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
-}
 
 // Logical tile id of this block with the XCD remap, or -1.
 __device__ __forceinline__ int64_t logical_tile(int64_t total, int64_t slot) {
@@ -126,8 +107,8 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
     return true;
 }
 
-// NW wavefronts per block: 4 (one per SIMD, wave tile 128 x 128) or 8 (two per SIMD, wave tile 128 x 64, so that
-// one wave's waits and memory instructions are covered by the other wave's MFMAs).
+// NW = 8 wavefronts per block, two per SIMD, wave tile 128 x 64: one wave's waits and memory instructions are covered by
+// the other wave's MFMAs.
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
@@ -209,11 +190,16 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             bmat = p.B0;
             brow0 = (int64_t)tc.n_tile * BN + wave * RPW;
         }
+        // weight rows past the last output column (an N that is not a multiple of the tile) re-read the last row;
+        // the columns they produce are never stored
+        if (brow0 > p.N - 1) brow0 = p.N - 1;
+        const int rel_max = (int)(p.N - 1 - brow0);
         b_base = (const char*)(bmat + (int64_t)tc.e * p.b_expert_stride + brow0 * p.ldb);
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
             const int r = wave * RPW + q * 8 + (lane >> 3);  // row of the LDS tile (fixes the swizzle)
-            b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.ldb * 2 + ((lane & 7) ^ swz(r)) * 16);
+            const int rel = q * 8 + (lane >> 3) < rel_max ? q * 8 + (lane >> 3) : rel_max;
+            b_off[q] = (uint32_t)(rel * (int)p.ldb * 2 + ((lane & 7) ^ swz(r)) * 16);
         }
     } else {
         b_step = BK * p.ldb * 2;
@@ -262,7 +248,6 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // kPrefetchDist k-steps ahead: the first half of the waves lines of the A slice, the second half lines of the B
     // slice.
     // ------------------------------------------------------------------------------------------
-    constexpr int kPrefetchDist = T::kBKMajor ? PICOMOE_PREFETCH_FWD : PICOMOE_PREFETCH_BWD;
     const char* pf_ptr;   // this lane's line at k-tile 0
     int64_t pf_step;      // bytes per k-tile
     {
@@ -288,9 +273,13 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             pf_step = b_step;
             if (MODE == kGateUp) {
                 const uint16_t* m = j < 128 ? p.B0 : p.B1;
-                pf_ptr = (const char*)(m + (int64_t)tc.e * p.b_expert_stride + ((int64_t)tc.n_tile * 128 + (j & 127)) * p.ldb) + half * 64;
+                int64_t wr = (int64_t)tc.n_tile * 128 + (j & 127);
+                wr = wr < p.N ? wr : p.N - 1;
+                pf_ptr = (const char*)(m + (int64_t)tc.e * p.b_expert_stride + wr * p.ldb) + half * 64;
             } else if (MODE == kDown) {
-                pf_ptr = (const char*)(p.B0 + (int64_t)tc.e * p.b_expert_stride + ((int64_t)tc.n_tile * BN + j) * p.ldb) + half * 64;
+                int64_t wr = (int64_t)tc.n_tile * BN + j;
+                wr = wr < p.N ? wr : p.N - 1;
+                pf_ptr = (const char*)(p.B0 + (int64_t)tc.e * p.b_expert_stride + wr * p.ldb) + half * 64;
             } else {
                 int64_t col = (int64_t)tc.n_tile * BN + (j & 3) * 64 + half * 32;
                 col = col + 8 <= p.N ? col : p.N - 8;
@@ -307,7 +296,6 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int pf_kt0 = kPrefetchDist < pf_n_kt ? kPrefetchDist : (pf_n_kt > 0 ? pf_n_kt - 1 : 0);
     const char* pf_cur = pf_ptr + (int64_t)pf_kt0 * pf_step + (pf_kt0 >= b_switch_kt ? pf_switch_delta : 0);
     auto prefetch_l2 = [&](int kt) {
-        if (kPrefetchDist == 0) return;
         // Destination v255: a register the kernel never allocates (it needs fewer than 255; the build checks the
         // generated code for any other mention of v255), so a load still in flight cannot land on a live value.
         asm volatile("global_load_dword v255, %0, off" ::"v"(pf_cur) : "v255", "memory");
@@ -510,8 +498,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 read_frags(kk, active);
                 if (kk == 3) {
                     // this wave's operand loads of the next k-tile have landed (its prefetch load may stay in flight)
-                    if (kPrefetchDist == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-                    else __builtin_amdgcn_s_waitcnt(0x0F71);
+                    __builtin_amdgcn_s_waitcnt(0x0F71);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 if (tail) mask_tail(kt, kk);
@@ -536,7 +523,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 phase_end();
             }
         };
-        constexpr int kUnroll = ((PICOMOE_KT_UNROLL_MODES >> MODE) & 1) ? PICOMOE_KT_UNROLL : 1;
+        constexpr int kUnroll = MODE == kWgrad ? 1 : kKtUnroll;
         const int n_plain = MODE == kWgrad ? n_kt - 1 : n_kt;  // k-steps without the tail mask
         int kt_done = 0;
         for (; kt_done + kUnroll <= n_plain; kt_done += kUnroll) {
@@ -551,7 +538,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // reads A fragments and issues MFMAs for those blocks only, and one whose 128 rows all lie past the end of a short tail
     // only loads and synchronises (same loads, waits and barriers, no reads, no MFMAs).  A tail tile then costs about what
     // its rows are worth instead of a half or a whole tile.
-    switch (PICOMOE_ROW_BLOCK_SKIP ? active_blocks : (active_blocks > 0 ? 4 : 0)) {
+    switch (active_blocks) {
         case 4: k_loop_pp(std::integral_constant<int, 4>{}); break;
         case 3: k_loop_pp(std::integral_constant<int, 3>{}); break;
         case 2: k_loop_pp(std::integral_constant<int, 2>{}); break;
@@ -636,12 +623,19 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 const float g = acc[i][j][r], u = acc[i][j + NJ / 2][r];
                 return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
             });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v; });
+            // (I is a multiple of 8: a 16-byte chunk lies inside the row or past its end as a whole)
+            for_chunks(i, [&](int trow, int c, u32x4_t v) {
+                if (col0 + c < I) *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v;
+            });
             if (p.out2) {
                 stage_block([&](int j, int r) { return acc[i][j][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) {
+                    if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v;
+                });
                 stage_block([&](int j, int r) { return acc[i][j + NJ / 2][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) {
+                    if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v;
+                });
             }
         }
     } else {
@@ -708,6 +702,7 @@ __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
     if (!locate_tile_slot(p.counts, p.E, p.n_tiles, g, xcd, g.full + t, &tc)) return;
     const float* w = p.ws + (int64_t)(xcd * kCusPerXcd + t * g.pieces) * (BM * BN);
     const int c4 = (threadIdx.x & 63) * 4;
+    if ((int64_t)tc.n_tile * BN + c4 >= p.N) return;  // columns past the output's last (N is a multiple of 8)
     for (int row = threadIdx.x >> 6; row < tc.rows; row += 4) {
         float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
         for (int pc = 0; pc < g.pieces; ++pc) {
@@ -747,13 +742,15 @@ MfmaParams base_params(const FfnShape& s) {
 int64_t ffn_mfma_workspace_bytes() { return kSplitWorkspaceBytes; }
 
 bool ffn_mfma_supported(const FfnShape& s) {
-    return s.dtype == PICOMOE_BF16 && s.H % 256 == 0 && s.I % 128 == 0 && s.H >= 256 && s.I >= 128;
+    // Both H and I are a contraction length somewhere (k-tiles of 64, no K tail except wgrad's); as output widths they
+    // only need whole 16-byte chunks, the tiles that reach past the last column clamp their loads and mask their stores.
+    return s.dtype == PICOMOE_BF16 && s.H % 64 == 0 && s.I % 64 == 0 && s.H >= 128 && s.I >= 128;
 }
 
 int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
                      hipStream_t st) {
     MfmaParams p = base_params(s);
-    p.K = s.H; p.N = s.I; p.n_tiles = (int)(s.I / 128);
+    p.K = s.H; p.N = s.I; p.n_tiles = (int)((s.I + 127) / 128);
     p.A = (const uint16_t*)x; p.lda = s.H;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;
     p.out = (uint16_t*)act; p.ldo = s.I; p.out2 = (uint16_t*)inter13;
@@ -764,7 +761,7 @@ int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const
 int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, void* ws,
                   int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
-    p.K = s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
+    p.K = s.I; p.N = s.H; p.n_tiles = (int)((s.H + BN - 1) / BN);
     p.A = (const uint16_t*)act; p.lda = s.I;
     p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;
     p.out = (uint16_t*)y; p.ldo = s.H; p.aux = (const uint16_t*)row_weight;
@@ -789,7 +786,7 @@ int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, co
 int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx, void* ws,
                      int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
-    p.K = 2 * s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
+    p.K = 2 * s.I; p.N = s.H; p.n_tiles = (int)((s.H + BN - 1) / BN);
     p.A = (const uint16_t*)d_inter13; p.lda = 2 * s.I;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;  // [K = I][N = H]
     p.out = (uint16_t*)dx; p.ldo = s.H;

@@ -16,13 +16,8 @@ constexpr int kNumXcd = 8;
 // and (row >> 1) & 7 puts the 8 row pairs on 8 different chunks: no bank conflicts (measured: 4 cycles per read).
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
-__device__ __forceinline__ void load16_to_lds(const void* g, char* l) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                     (__attribute__((address_space(3))) void*)l, 16, 0, 0);
-}
-
-// The same load as an instruction sequence the compiler does not look into: wave-uniform base pointer plus a 32-bit
-// byte offset per lane, LDS destination (wave-uniform, lane l lands at +16*l) through M0.  Why: the compiler's
+// A 16-byte direct-to-LDS load as an instruction sequence the compiler does not look into: wave-uniform base pointer plus
+// a 32-bit byte offset per lane, LDS destination (wave-uniform, lane l lands at +16*l) through M0.  Why: the compiler's
 // wait-count pass knows a builtin direct-to-LDS load is in flight and puts "s_waitcnt vmcnt(0)" in front of every later
 // LDS read it cannot prove disjoint from the destination -- it does so for the transpose reads
 // (__builtin_amdgcn_ds_read_tr16_b64), which then wait for loads issued a moment ago.  A kernel that uses this form

@@ -12,6 +12,8 @@ is the epilogue of the gate/up GEMM, silu-mul-backward is the epilogue of the ``
 autograd path keeps ``[g|u]`` from the forward instead of recomputing it.
 """
 
+import collections
+
 import torch
 import torch.nn.functional as F
 
@@ -92,18 +94,31 @@ def _gate_up_fp8(xq, x_scale, counts, gate_q, gate_scale, up_q, up_scale, keep_i
     return act, inter13
 
 
-_workspaces = {}
+_workspaces = collections.OrderedDict()
+_MAX_WORKSPACES = 4
 
 
 def _ffn_workspace(device):
     """Scratch for the split last round of the down / dgrad_x kernels (picomoe_ffn_workspace_bytes, 64 MB): one buffer
-    per device and stream, allocated on first use -- kernels of one stream run one after the other, so they can share it."""
+    per device and stream, allocated on first use -- kernels of one stream run one after the other, so they can share it.
+    At most ``_MAX_WORKSPACES`` buffers are kept; when a further stream asks for one, the least recently used goes back
+    to the caching allocator, which hands it out again only on the stream it was allocated and used on, i.e. in order
+    behind the kernels that still read it."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None:
+        while len(_workspaces) >= _MAX_WORKSPACES:
+            _workspaces.popitem(last=False)
         ws = torch.empty(_lib.load().picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
+    else:
+        _workspaces.move_to_end(key)
     return ws
+
+
+def release_workspaces():
+    """Drops every cached split-round workspace (64 MB per device and stream that has run an expert FFN)."""
+    _workspaces.clear()
 
 
 def _down(act, counts, down_w, row_weight):

@@ -124,9 +124,12 @@ def test_explicit_dgrad_wgrad_api(gpu, dtype):
         assert torch.allclose(got.cpu().float(), want, **tol)
 
 
-@pytest.mark.parametrize("H,I,counts", [(256, 512, [130, 128, 126, 0, 1, 64, 63, 0]), (100, 36, [7, 300]), (256, 384, [300, 0, 5, 257]), (512, 128, [1, 1000, 70])])
+@pytest.mark.parametrize("H,I,counts", [(256, 512, [130, 128, 126, 0, 1, 64, 63, 0]), (100, 36, [7, 300]), (256, 384, [300, 0, 5, 257]), (512, 128, [1, 1000, 70]),
+                                        (320, 192, [300, 0, 5, 257]), (128, 448, [129, 64, 1]), (704, 320, [33, 520, 0, 256]), (192, 128, [257, 3])])
 def test_bf16_ragged_against_oracle(gpu, H, I, counts):
-    """bf16: outputs and gradients within rtol 1e-2 of the oracle (measured against the magnitude of each tensor)."""
+    """bf16: outputs and gradients within rtol 1e-2 of the oracle (measured against the magnitude of each tensor).
+    The last four shapes are widths the 256-column tiles do not divide (hidden 320, 128, 704, 192; FFN 192, 448, 320): the
+    MFMA kernels run them with clamped loads and masked stores in the last tile column."""
     from picotron_amd.expert_parallel import megakernel
 
     E = len(counts)
@@ -142,8 +145,9 @@ def test_bf16_ragged_against_oracle(gpu, H, I, counts):
         assert (got.cpu().float() - want).abs().max() <= 1e-2 * want.abs().max()
 
 
+@pytest.mark.parametrize("H", [512, 320])
 @pytest.mark.parametrize("counts", [[300, 260, 100, 515], [256, 512, 7, 129], [40, 0, 3, 1]])
-def test_split_last_round_matches_whole_tiles(gpu, counts):
+def test_split_last_round_matches_whole_tiles(gpu, counts, H):
     """With a workspace the down and dgrad_x kernels cut the tiles of the last, partly filled round into 2 or 4 ranges of K
     (K here is 32 and 64 k-tiles, enough for 2 and 4 pieces) and add the fp32 partial tiles up in a second kernel: the
     result must agree with the whole-tile kernels to the rounding of the partial sums, and with the oracle at the bf16
@@ -151,7 +155,7 @@ def test_split_last_round_matches_whole_tiles(gpu, counts):
     from picotron_amd import _lib
     from picotron_amd.expert_parallel import megakernel as mk
 
-    E, H, I = len(counts), 512, 2048
+    E, I = len(counts), 2048
     x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.bfloat16, 11, scale=0.03)
     N = x.shape[0]
     act = (torch.randn(N, I, generator=g) * 0.5).bfloat16().cuda()
@@ -187,12 +191,13 @@ def test_split_last_round_matches_whole_tiles(gpu, counts):
         assert torch.equal(fn(ws).float().cpu(), split)               # fixed summation order: run to run identical
 
 
-@pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32)])
+@pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (320, 192, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32)])
 def test_rows_past_the_segments_are_never_read_into_a_result(gpu, H, I, dtype):
     """n_rows > sum(counts), as in the capacity modes where the buffers are sized for every routed row and only the kept
     rows are laid out: the slack rows of every input hold NaN, the slack rows of every output are pre-filled.  Results
     for the valid rows and all three weight gradients must equal the run without slack bit for bit, and the slack rows
-    of the outputs must come back untouched.  Covers the MFMA kernels (hidden 256) and the generic ones."""
+    of the outputs must come back untouched.  Covers the MFMA kernels (hidden 256; hidden 320 / FFN 192 with a partly
+    filled last tile column) and the generic ones."""
     from picotron_amd import _lib
 
     lib = _lib.load()
@@ -283,3 +288,19 @@ def test_mlp_module_runs_the_kernels(gpu):
     assert y.shape == (3, 5, 32) and torch.allclose(y.cpu(), want, atol=1e-5)
     y.sum().backward()
     assert all(p.grad is not None for p in m.parameters())
+
+
+def test_workspace_cache_is_bounded(gpu):
+    """The split-round workspaces are cached per stream; the cache keeps at most four and can be emptied."""
+    from picotron_amd.expert_parallel import megakernel as mk
+
+    mk.release_workspaces()
+    dev = torch.device("cuda", torch.cuda.current_device())
+    first = mk._ffn_workspace(dev)
+    assert mk._ffn_workspace(dev) is first                     # same stream: same buffer
+    for _ in range(6):
+        with torch.cuda.stream(torch.cuda.Stream()):
+            mk._ffn_workspace(dev)
+    assert len(mk._workspaces) == mk._MAX_WORKSPACES
+    mk.release_workspaces()
+    assert len(mk._workspaces) == 0
