@@ -151,15 +151,27 @@ class GemmTimer:
         return {k: (v["ms"] / v["n"], v["flop"], v["n"]) for k, v in per.items()}
 
 
+def outlier_activation(n, h, device, seed):
+    """[n, h] bf16 ~ N(0, 1) with 0.1 % of the entries replaced by outliers ~ N(0, 50): the data of the FP8 round-trip
+    configuration."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn(n, h, generator=g, device=device)
+    mask = torch.rand(n, h, generator=g, device=device) < 0.001
+    return torch.where(mask, 50.0 * torch.randn(n, h, generator=g, device=device), x).bfloat16()
+
+
 def fp8_quant_bandwidth(device, n=16384, h=4096, sets=6, iters=60):
-    """FP8 E4M3 dispatch quantise at 16384 x 4096 bf16, rotating over buffer sets larger than the 256 MB
-    last-level cache so the figure is HBM traffic.  Returns (GB/s quantise, GB/s dequantise)."""
+    """FP8 E4M3 dispatch quantise at 16384 x 4096 bf16 on the round-trip configuration's data (0.1 % outliers of
+    50 sigma), rotating over buffer sets larger than the 256 MB last-level cache so the figure is HBM traffic.
+    Returns (GB/s quantise, GB/s dequantise, us quantise, us dequantise)."""
     import torch
 
     from picotron_amd import _lib
 
     lib = _lib.load()
-    xs = [torch.randn(n, h, device=device).bfloat16() for _ in range(sets)]
+    xs = [outlier_activation(n, h, device, seed) for seed in range(sets)]
     qs = [torch.empty(n, h, dtype=torch.uint8, device=device) for _ in range(sets)]
     ss = [torch.empty(n, dtype=torch.float32, device=device) for _ in range(sets)]
     os_ = [torch.empty(n, h, dtype=torch.bfloat16, device=device) for _ in range(sets)]
@@ -181,55 +193,77 @@ def fp8_quant_bandwidth(device, n=16384, h=4096, sets=6, iters=60):
 
 
 def fp8_gemm_variant(moe, step, w, steps):
-    """The same layer step with the forward gate/up GEMM on FP8 MFMA (E4M3 dispatch codes x per-row quantised weights,
-    re-quantised every step as in training): step time, and the FP8 kernel and the weight quantiser timed with events."""
+    """The same layer step with the forward GEMMs on FP8 MFMA (E4M3 dispatch codes x per-row quantised weights,
+    re-quantised every step as in training): first gate/up alone, then gate/up and down (the SwiGLU output quantised per
+    row by one more pass).  Step times, and the FP8 kernels and the quantisers timed with events."""
     import torch
 
     from picotron_amd.expert_parallel import megakernel as mk
 
-    times = {"gate_up_fp8": [], "quantize_weights": []}
-    pool = [torch.cuda.Event(enable_timing=True) for _ in range(2 * 3 * steps + 8)]
-    state = {"on": False}
+    names = ("_gate_up_fp8", "_down_fp8", "quantize_expert_weights", "_quantize_rows")
+    orig = {n: getattr(mk, n) for n in names}
+    state = {"on": False, "times": None, "pool": []}
 
     def wrap(name, fn):
         def timed(*a, **kw):
-            if not state["on"] or len(pool) < 2:
+            if not state["on"] or len(state["pool"]) < 2:
                 return fn(*a, **kw)
-            st, en = pool.pop(), pool.pop()
+            st, en = state["pool"].pop(), state["pool"].pop()
             st.record()
             out = fn(*a, **kw)
             en.record()
-            times[name].append((st, en))
+            state["times"][name].append((st, en))
             return out
         return timed
 
-    orig = (mk._gate_up_fp8, mk.quantize_expert_weights)
-    mk._gate_up_fp8 = wrap("gate_up_fp8", mk._gate_up_fp8)
-    mk.quantize_expert_weights = wrap("quantize_weights", mk.quantize_expert_weights)
-    moe.ep_fp8_gemm = True
+    for n in names:
+        setattr(mk, n, wrap(n, orig[n]))
+    rows = w["T"] * w["k"]
+    out = {}
     try:
-        for _ in range(3):
-            step()
-        torch.cuda.synchronize()
-        state["on"] = True
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / steps
+        for mode in (True, "all"):
+            moe.ep_fp8_gemm = mode
+            state["times"] = {n: [] for n in names}
+            state["pool"] = [torch.cuda.Event(enable_timing=True) for _ in range(2 * 6 * steps + 8)]
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+            state["on"] = True
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / steps
+            state["on"] = False
+            per_call = lambda n: sum(a.elapsed_time(b) for a, b in state["times"][n]) / max(len(state["times"][n]), 1)
+            per_step = lambda n: sum(a.elapsed_time(b) for a, b in state["times"][n]) / max(steps, 1)
+            gu_ms, q_ms = per_call("_gate_up_fp8"), per_step("quantize_expert_weights")
+            gu_flop = 4.0 * rows * w["H"] * w["I"]
+            if mode is True:
+                log(f"[bench] fp8 gate/up GEMM variant: {ms:.3f} ms/step, gate_up_fp8 {gu_ms:.2f} ms ({gu_flop / gu_ms / 1e9:.0f} TFLOP/s), "
+                    f"weight quantisation {q_ms:.2f} ms/step")
+                out = {"ms_per_step": ms, "tokens_per_s": w["T"] / (ms * 1e-3), "gate_up_fp8_ms": gu_ms,
+                       "gate_up_fp8_tflops": gu_flop / gu_ms / 1e9, "frac_fp8_mfma_peak": gu_flop / gu_ms / 1e9 / 5000.0,
+                       "weight_quant_ms_per_step": q_ms,
+                       "note": "forward gate/up on v_mfma_f32_32x32x64_f8f6f4; down, dgrad and wgrad stay bf16; not the headline value"}
+            else:
+                # _down_fp8 = the row quantiser of the SwiGLU output + the FP8 down kernel; the kernel alone is the difference
+                d_ms, aq_ms = per_call("_down_fp8"), per_call("_quantize_rows")
+                k_ms = d_ms - aq_ms
+                d_flop = 2.0 * rows * w["H"] * w["I"]
+                log(f"[bench] fp8 gate/up + down GEMM variant: {ms:.3f} ms/step, down_fp8 {k_ms:.2f} ms ({d_flop / k_ms / 1e9:.0f} TFLOP/s) "
+                    f"+ {aq_ms:.2f} ms quantising its input, weight quantisation {q_ms:.2f} ms/step")
+                out["all"] = {"ms_per_step": ms, "tokens_per_s": w["T"] / (ms * 1e-3), "gate_up_fp8_ms": gu_ms,
+                              "down_fp8_ms": k_ms, "down_fp8_tflops": d_flop / k_ms / 1e9,
+                              "down_frac_fp8_mfma_peak": d_flop / k_ms / 1e9 / 5000.0, "act_quant_ms": aq_ms,
+                              "weight_quant_ms_per_step": q_ms,
+                              "note": "forward gate/up and down on FP8 MFMA (SwiGLU output quantised per row); dgrad and wgrad stay bf16"}
     finally:
         state["on"] = False
         moe.ep_fp8_gemm = False
-        mk._gate_up_fp8, mk.quantize_expert_weights = orig
-    k_ms = sum(a.elapsed_time(b) for a, b in times["gate_up_fp8"]) / max(len(times["gate_up_fp8"]), 1)
-    q_ms = sum(a.elapsed_time(b) for a, b in times["quantize_weights"]) / max(steps, 1)  # two calls (gate, up) per step
-    flop = 4.0 * w["T"] * w["k"] * w["H"] * w["I"]
-    log(f"[bench] fp8 gate/up GEMM variant: {ms:.3f} ms/step, gate_up_fp8 {k_ms:.2f} ms ({flop / k_ms / 1e9:.0f} TFLOP/s), "
-        f"weight quantisation {q_ms:.2f} ms/step")
-    return {"ms_per_step": ms, "tokens_per_s": w["T"] / (ms * 1e-3), "gate_up_fp8_ms": k_ms,
-            "gate_up_fp8_tflops": flop / k_ms / 1e9, "frac_fp8_mfma_peak": flop / k_ms / 1e9 / 5000.0,
-            "weight_quant_ms_per_step": q_ms,
-            "note": "forward gate/up on v_mfma_f32_32x32x64_f8f6f4; down, dgrad and wgrad stay bf16; not the headline value"}
+        for n in names:
+            setattr(mk, n, orig[n])
+    return out
 
 
 def cpu_baseline(w, moe, budget_s=25.0):
@@ -310,13 +344,7 @@ def fp8_bench(args):
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device = torch.device("cuda:0")
     n, h, sets = 16384, 4096, 6
-    g = torch.Generator(device=device).manual_seed(0)
-    xs = []
-    for _ in range(sets):
-        x = torch.randn(n, h, generator=g, device=device)
-        mask = torch.rand(n, h, generator=g, device=device) < 0.001
-        xs.append(torch.where(mask, 50.0 * torch.randn(n, h, generator=g, device=device), x).bfloat16())
-        del x, mask
+    xs = [outlier_activation(n, h, device, seed) for seed in range(sets)]
     qs = [torch.empty(n, h, dtype=torch.uint8, device=device) for _ in range(sets)]
     ss = [torch.empty(n, dtype=torch.float32, device=device) for _ in range(sets)]
     ys = [torch.empty(n, h, dtype=torch.bfloat16, device=device) for _ in range(sets)]
@@ -552,7 +580,7 @@ def main():
         qg, dg, tq, td = fp8_quant_bandwidth(device)
         result["fp8_quant"] = {"GBps": qg, "frac_hbm": qg / HBM_PEAK_GBPS, "us": tq, "dequant_GBps": dg,
                                "dequant_frac_hbm": dg / HBM_PEAK_GBPS, "dequant_us": td,
-                               "shape": "16384 x 4096 bf16 -> e4m3 + fp32 scale, 201392128 B per pass"}
+                               "shape": "16384 x 4096 bf16 (N(0,1), 0.1 % outliers of 50 sigma) -> e4m3 + fp32 scale, 201392128 B per pass"}
         log(f"[bench] fp8 quant {qg:.0f} GB/s ({tq:.1f} us), dequant {dg:.0f} GB/s ({td:.1f} us)")
 
     if w["fp8"] and not args.no_kernel_times:

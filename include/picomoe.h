@@ -28,7 +28,7 @@ extern "C" {
 #define PICOMOE_F32 0
 #define PICOMOE_BF16 1
 
-#define PICOMOE_ABI_VERSION 3
+#define PICOMOE_ABI_VERSION 4
 
 /* ABI version of the loaded library (compare with PICOMOE_ABI_VERSION). */
 int picomoe_abi_version(void);
@@ -145,6 +145,14 @@ int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, const int64_t*
 int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden, int64_t inter,
                      const void* down_w, const void* row_weight, int dtype, void* y, void* workspace, int64_t workspace_bytes,
                      void* stream);
+/* The same down GEMM on FP8 MFMA: actq [n_rows, inter] E4M3 codes of the SwiGLU output with one fp32 scale per row
+ * (picomoe_fp8_quant of act), down_wq [E, hidden, inter] codes with one fp32 scale per output row ([E * hidden]);
+ * y [n_rows, hidden] bf16 = (actq . down_wq[e]^T) * act_scale * down_scale, fp32 accumulation, times the optional bf16
+ * row_weight as in picomoe_ffn_down (EP/megakernel.py:305, :95-96).  hidden % 256 == 0 and inter % 128 == 0, else
+ * PICOMOE_ERR_ARG.  No counterpart in the reference (it has no FP8 GEMM): compared with the bf16 GEMM at rtol 5e-2. */
+int picomoe_ffn_down_fp8(const void* actq, const float* act_scale, const int64_t* counts, int num_experts, int64_t n_rows,
+                         int64_t hidden, int64_t inter, const void* down_wq, const float* down_scale, const void* row_weight,
+                         void* y, void* stream);
 /* Replaces da = dy @ down_w[e] and _silu_and_mul_bwd (EP/megakernel.py:344-345, :187-197) in one kernel:
  * d_inter13 [n_rows, 2*inter] = [dg | du]; act_out (optional) = silu(g) * u rebuilt from inter13. */
 int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,

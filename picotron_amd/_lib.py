@@ -12,7 +12,7 @@ import torch
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libpicomoe.so")
 HEADER_PATH = os.path.join(os.path.dirname(_PKG_DIR), "include", "picomoe.h")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -38,6 +38,7 @@ _SIGNATURES = {
     "picomoe_combine_bwd": [_p, _p, _p, _p, _i64, _i32, _i64, _i32, _p, _p, _p],
     "picomoe_ffn_gate_up": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
     "picomoe_ffn_gate_up_fp8": [_p, _p, _p, _i32, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
+    "picomoe_ffn_down_fp8": [_p, _p, _p, _i32, _i64, _i64, _i64, _p, _p, _p, _p, _p],
     "picomoe_ffn_down": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _i64, _p],
     "picomoe_ffn_dgrad_act": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
     "picomoe_ffn_dgrad_x": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _i64, _p],

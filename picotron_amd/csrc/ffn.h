@@ -43,10 +43,14 @@ int64_t ffn_mfma_workspace_bytes();
 int ffn_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, int64_t P, int64_t Q,
                    void* out, hipStream_t st);
 
-// FP8 (E4M3) MFMA gate/up: codes + one fp32 scale per activation row and per weight row (ffn_fp8.hip)
+// FP8 (E4M3) MFMA gate/up and down: codes + one fp32 scale per activation row and per weight row (ffn_fp8.hip)
 bool ffn_fp8_supported(const FfnShape& s);
 int ffn_fp8_gate_up(const FfnShape& s, const void* xq, const float* x_scale, const void* gq, const void* uq,
                     const float* g_scale, const float* u_scale, void* act, void* inter13, hipStream_t st);
+
+// FP8 MFMA down: act codes + one fp32 scale per row, down_w codes + one scale per output row; y bf16 (* row_weight)
+int ffn_fp8_down(const FfnShape& s, const void* actq, const float* act_scale, const void* dq, const float* d_scale,
+                 const void* row_weight, void* y, hipStream_t st);
 
 // SwiGLU pieces shared by both families (fp32 arithmetic on values already rounded to the storage type).
 __device__ __forceinline__ float sigmoid_f32(float g) { return 1.0f / (1.0f + expf(-g)); }

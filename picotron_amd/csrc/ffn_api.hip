@@ -34,6 +34,17 @@ extern "C" int picomoe_ffn_gate_up_fp8(const void* xq, const float* x_scale, con
     return ffn_fp8_gate_up(s, xq, x_scale, gate_wq, up_wq, gate_scale, up_scale, act, inter13, (hipStream_t)stream);
 }
 
+extern "C" int picomoe_ffn_down_fp8(const void* actq, const float* act_scale, const int64_t* counts, int num_experts,
+                                    int64_t n_rows, int64_t hidden, int64_t inter, const void* down_wq,
+                                    const float* down_scale, const void* row_weight, void* y, void* stream) {
+    FfnShape s;
+    PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, PICOMOE_BF16));
+    PICOMOE_CHECK_ARG(ffn_fp8_supported(s));
+    if (n_rows == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(actq && act_scale && down_wq && down_scale && y);
+    return ffn_fp8_down(s, actq, act_scale, down_wq, down_scale, row_weight, y, (hipStream_t)stream);
+}
+
 extern "C" int64_t picomoe_ffn_workspace_bytes(void) { return ffn_mfma_workspace_bytes(); }
 
 extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,

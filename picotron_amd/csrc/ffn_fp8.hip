@@ -1,7 +1,8 @@
-// FP8 (E4M3) MFMA kernel for the gate/up projection of the expert FFN on gfx950 (MI355X): the per-token quantised
-// activations of the FP8 dispatch (codes + one fp32 scale per row) meet expert weights quantised the same way
-// (one scale per output row) in v_mfma_f32_32x32x64_f8f6f4, fp32 accumulation, and the two scales are applied to
-// the accumulators in the epilogue, fused with SwiGLU.
+// FP8 (E4M3) MFMA kernels for the forward projections of the expert FFN on gfx950 (MI355X): per-row quantised
+// activations (codes + one fp32 scale per row: the FP8 dispatch's rows for gate/up, the quantised SwiGLU output for
+// down) meet expert weights quantised the same way (one scale per output row) in v_mfma_f32_32x32x64_f8f6f4, fp32
+// accumulation, and the two scales are applied to the accumulators in the epilogue -- fused with SwiGLU for gate/up,
+// with the optional row weight for down.
 //
 // Same frame as the bf16 kernels: 256 x 256 block tile, 8 wavefronts (two per SIMD) of 128 x 64, two 64 KB LDS
 // stages filled by 16-byte direct-to-LDS loads.  A 128-byte LDS row now holds 128 k values, so one k-step is two
@@ -20,22 +21,28 @@ constexpr int kFp8BK = 128;  // k values (bytes) per k-step
 
 typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 
+enum Fp8Mode { kFp8GateUp = 0, kFp8Down = 1 };
+
 struct Fp8Params {
     const int64_t* counts;
     int E;
-    int64_t n_rows, H, I;
+    int64_t n_rows;
+    int64_t K;             // contraction length: H (gate/up) or I (down); row pitch in bytes of both operands
+    int64_t N;             // output columns: I (gate/up) or H (down); weight rows per expert and matrix
     int n_tiles;
-    const uint8_t* xq;     // [n_rows, H] e4m3 codes
+    const uint8_t* xq;     // [n_rows, K] e4m3 codes
     const float* x_scale;  // [n_rows]
-    const uint8_t* gq;     // [E, I, H]
-    const uint8_t* uq;
-    const float* g_scale;  // [E * I]
+    const uint8_t* gq;     // gate/up: gate_w codes [E, I, H]; down: down_w codes [E, H, I]
+    const uint8_t* uq;     // gate/up: up_w codes; down: unused
+    const float* g_scale;  // [E * N]
     const float* u_scale;
-    uint16_t* act;      // [n_rows, I] bf16
-    uint16_t* inter13;  // [n_rows, 2I] bf16 or null
+    uint16_t* act;         // gate/up: act [n_rows, I] bf16; down: y [n_rows, H] bf16
+    uint16_t* inter13;     // gate/up: [n_rows, 2I] bf16 or null
+    const uint16_t* row_weight;  // down: optional bf16 [n_rows], multiplied into the rounded output
 };
 
-__global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8Params p) {
+template <int MODE>
+__global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p) {
     constexpr int NI = 4, NJ = 2, kWaveCols = 4, CW = 64, QN = 4, RPW = 32;
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
@@ -45,21 +52,23 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
     const int l31 = lane & 31, hi = lane >> 5;
-    const int n_kt = (int)(p.H / kFp8BK);
+    const int n_kt = (int)(p.K / kFp8BK);
     const bool wave_active = wm * 128 < tc.rows;
 
-    // global -> LDS: wave w fills rows [32w, 32w + 32) of both tiles, 8 rows (128 B each) per instruction.  B tile:
-    // per wave column (64 rows) 32 gate rows then 32 up rows of the same FFN columns: even waves load gate rows.
+    // global -> LDS: wave w fills rows [32w, 32w + 32) of both tiles, 8 rows (128 B each) per instruction.  B tile,
+    // gate/up: per wave column (64 rows) 32 gate rows then 32 up rows of the same FFN columns: even waves load gate rows;
+    // down: 256 consecutive rows of down_w[e].
     uint32_t a_off[QN], b_off[QN];
-    const char* a_base = (const char*)(p.xq + tc.row0 * p.H);
-    const uint8_t* bmat = (wave & 1) ? p.uq : p.gq;
-    const char* b_base = (const char*)(bmat + ((int64_t)tc.e * p.I + (int64_t)tc.n_tile * 128 + (wave >> 1) * 32) * p.H);
+    const char* a_base = (const char*)(p.xq + tc.row0 * p.K);
+    const uint8_t* bmat = MODE == kFp8GateUp && (wave & 1) ? p.uq : p.gq;
+    const int64_t brow0 = MODE == kFp8GateUp ? (int64_t)tc.n_tile * 128 + (wave >> 1) * 32 : (int64_t)tc.n_tile * BN + wave * RPW;
+    const char* b_base = (const char*)(bmat + ((int64_t)tc.e * p.N + brow0) * p.K);
 #pragma unroll
     for (int q = 0; q < QN; ++q) {
         const int r = wave * RPW + q * 8 + (lane >> 3);
         const int ar = r < tc.rows ? r : tc.rows - 1;  // rows past the segment re-read its last row (never stored)
-        a_off[q] = (uint32_t)(ar * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
-        b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.H + ((lane & 7) ^ swz(r)) * 16);
+        a_off[q] = (uint32_t)(ar * (int)p.K + ((lane & 7) ^ swz(r)) * 16);
+        b_off[q] = (uint32_t)((q * 8 + (lane >> 3)) * (int)p.K + ((lane & 7) ^ swz(r)) * 16);
     }
     // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt.  Opaque loads: the waits between
     // a load and the LDS reads of its data are the explicit ones below (prologue, k-loop barrier, end of the loop).
@@ -179,26 +188,24 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
-    // epilogue: scale, round g and u to bf16 (what the two Linear outputs of the reference hold), SwiGLU, and stage
-    // 32 rows at a time through a wave-private slice of LDS so that the stores are 16-byte lanes of contiguous rows
+    // epilogue: the two scales, rounding to bf16, and 32 rows at a time through a wave-private slice of LDS so that the
+    // stores are 16-byte lanes of contiguous rows
     float* row_scale = (float*)(lds + kStageBytes);  // 256 floats, past the staging slices
     if (tid < BM) row_scale[tid] = p.x_scale[tc.row0 + (tid < tc.rows ? tid : tc.rows - 1)];
-    const int64_t I = p.I;
-    const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
-    const float gs = p.g_scale[(int64_t)tc.e * I + col0 + l31], us = p.u_scale[(int64_t)tc.e * I + col0 + l31];
-    __syncthreads();
-    constexpr int kEpiCols = CW / 2;
+    constexpr int kEpiCols = MODE == kFp8GateUp ? CW / 2 : CW;
     constexpr int kEpiStride = (kEpiCols + 8) * 2;
     char* epi = lds + wave * (32 * kEpiStride);
     constexpr int kChunksPerRow = kEpiCols / 8;
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
-    auto stage_block = [&](auto value) {
+    auto stage_block = [&](auto value) {  // value(j, r), j over the 32-column blocks of a pass
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
-            *(uint16_t*)(epi + row * kEpiStride + l31 * 2) = (uint16_t)f32_to_bf16_bits(value(r));
-        }
+        for (int j = 0; j < kEpiCols / 32; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
+                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + l31) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
+            }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
     auto for_chunks = [&](int i, auto f) {
@@ -211,24 +218,56 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_gate_up_kernel(Fp8P
             if (trow < tc.rows) f(trow, ch * 8, v);
         }
     };
+    if (MODE == kFp8GateUp) {
+        // g and u rounded to bf16 (what the two Linear outputs of the reference hold), then SwiGLU
+        const int64_t I = p.N;
+        const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
+        const float gs = p.g_scale[(int64_t)tc.e * I + col0 + l31], us = p.u_scale[(int64_t)tc.e * I + col0 + l31];
+        __syncthreads();
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < NI; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float sx = row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)];
-            acc[i][0][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][r] * sx * gs));
-            acc[i][1][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][r] * sx * us));
+            for (int r = 0; r < 16; ++r) {
+                const float sx = row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)];
+                acc[i][0][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][r] * sx * gs));
+                acc[i][1][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][r] * sx * us));
+            }
+            stage_block([&](int, int r) {
+                const float g = acc[i][0][r], u = acc[i][1][r];
+                return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
+            });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.act + (tc.row0 + trow) * I + col0 + c) = v; });
+            if (p.inter13) {
+                stage_block([&](int, int r) { return acc[i][0][r]; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + col0 + c) = v; });
+                stage_block([&](int, int r) { return acc[i][1][r]; });
+                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + I + col0 + c) = v; });
+            }
         }
-        stage_block([&](int r) {
-            const float g = acc[i][0][r], u = acc[i][1][r];
-            return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
-        });
-        for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.act + (tc.row0 + trow) * I + col0 + c) = v; });
-        if (p.inter13) {
-            stage_block([&](int r) { return acc[i][0][r]; });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + col0 + c) = v; });
-            stage_block([&](int r) { return acc[i][1][r]; });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + I + col0 + c) = v; });
+    } else {
+        // y = bf16(acc * row scale * column scale), times the row weight (rounded again) when there is one
+        const int64_t H = p.N;
+        const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
+        float ws[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) ws[j] = p.g_scale[(int64_t)tc.e * H + col0 + j * 32 + l31];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            if (wm * 128 + i * 32 >= tc.rows) continue;  // wave-uniform
+            stage_block([&](int j, int r) {
+                return acc[i][j][r] * row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)] * ws[j];
+            });
+            for_chunks(i, [&](int trow, int c, u32x4_t v) {
+                const int64_t grow = tc.row0 + trow;
+                if (p.row_weight) {
+                    const float rw = bf16_bits_to_f32(p.row_weight[grow]);
+#pragma unroll
+                    for (int w2 = 0; w2 < 4; ++w2)
+                        v[w2] = pack_bf16x2(__uint_as_float(v[w2] << 16) * rw, __uint_as_float(v[w2] & 0xFFFF0000u) * rw);
+                }
+                *(u32x4_t*)(p.act + grow * H + col0 + c) = v;
+            });
         }
     }
 }
@@ -240,10 +279,21 @@ bool ffn_fp8_supported(const FfnShape& s) { return s.H % 256 == 0 && s.I % 128 =
 int ffn_fp8_gate_up(const FfnShape& s, const void* xq, const float* x_scale, const void* gq, const void* uq,
                     const float* g_scale, const float* u_scale, void* act, void* inter13, hipStream_t st) {
     Fp8Params p{};
-    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.H = s.H; p.I = s.I; p.n_tiles = (int)(s.I / 128);
+    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.K = s.H; p.N = s.I; p.n_tiles = (int)(s.I / 128);
     p.xq = (const uint8_t*)xq; p.x_scale = x_scale;
     p.gq = (const uint8_t*)gq; p.uq = (const uint8_t*)uq; p.g_scale = g_scale; p.u_scale = u_scale;
     p.act = (uint16_t*)act; p.inter13 = (uint16_t*)inter13;
-    hipLaunchKernelGGL(ffn_fp8_gate_up_kernel, dim3(grid_m_grouped(s, p.n_tiles)), dim3(kFp8Waves * 64), 0, st, p);
+    hipLaunchKernelGGL(ffn_fp8_kernel<kFp8GateUp>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(kFp8Waves * 64), 0, st, p);
+    return picomoe_launch_status();
+}
+
+int ffn_fp8_down(const FfnShape& s, const void* actq, const float* act_scale, const void* dq, const float* d_scale,
+                 const void* row_weight, void* y, hipStream_t st) {
+    Fp8Params p{};
+    p.counts = s.counts; p.E = s.E; p.n_rows = s.n_rows; p.K = s.I; p.N = s.H; p.n_tiles = (int)(s.H / BN);
+    p.xq = (const uint8_t*)actq; p.x_scale = act_scale;
+    p.gq = (const uint8_t*)dq; p.g_scale = d_scale;
+    p.act = (uint16_t*)y; p.row_weight = (const uint16_t*)row_weight;
+    hipLaunchKernelGGL(ffn_fp8_kernel<kFp8Down>, dim3(grid_m_grouped(s, p.n_tiles)), dim3(kFp8Waves * 64), 0, st, p);
     return picomoe_launch_status();
 }

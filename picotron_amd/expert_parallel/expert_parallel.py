@@ -82,7 +82,8 @@ class MoELayer(nn.Module):
         self.ep_backend = getattr(config, "ep_backend", "torch")
         self.ep_fp8_dispatch = getattr(config, "ep_fp8_dispatch", False)
         # not in the reference: with the FP8 dispatch on, feed the forward gate/up GEMM with the E4M3 codes on FP8 MFMA
-        # (weights quantised per output row) instead of the dequantised rows on bf16 MFMA
+        # (weights quantised per output row) instead of the dequantised rows on bf16 MFMA; "all" also runs the forward
+        # down GEMM on FP8 MFMA (SwiGLU output quantised per row).  The backward is bf16 either way.
         self.ep_fp8_gemm = getattr(config, "ep_fp8_gemm", False)
         self._fp8_weights = None
 
@@ -235,16 +236,20 @@ class MoELayer(nn.Module):
                 and megakernel.fp8_gemm_supported(self.expert_dim, self.local_experts[0].gate_proj.weight.shape[0]))
 
     def _quantized_weights(self):
-        """E4M3 codes + per-row scales of the stacked gate / up weights.  Training: redone every forward (the
+        """E4M3 codes + per-row scales of the stacked gate / up (and, with ``ep_fp8_gemm == "all"``, down) weights.  Training: redone every forward (the
         optimizer changes the weights every step).  Eval: kept until a parameter's version counter moves; after a
         write that bypasses the counters (``p.data``) call ``invalidate_fp8_weights``."""
-        gates, ups, _ = self._expert_params()
-        key = (self._stacks[0].data_ptr(), self._stacks[1].data_ptr(), tuple(p._version for p in gates + ups))
+        gates, ups, downs = self._expert_params()
+        with_down = self.ep_fp8_gemm == "all"
+        params = gates + ups + (downs if with_down else [])
+        key = (with_down, self._stacks[0].data_ptr(), self._stacks[1].data_ptr(), self._stacks[2].data_ptr(),
+               tuple(p._version for p in params))
         if self.training or self._fp8_weights is None or self._fp8_weights[0] != key:
             with torch.no_grad():
-                gq, gs = megakernel.quantize_expert_weights(self._stacks[0])
-                uq, us = megakernel.quantize_expert_weights(self._stacks[1])
-            self._fp8_weights = (key, (gq, gs, uq, us))
+                quantized = megakernel.quantize_expert_weights(self._stacks[0]) + megakernel.quantize_expert_weights(self._stacks[1])
+                if with_down:
+                    quantized += megakernel.quantize_expert_weights(self._stacks[2])
+            self._fp8_weights = (key, quantized)
         return self._fp8_weights[1]
 
     def invalidate_fp8_weights(self):

@@ -94,6 +94,35 @@ def _gate_up_fp8(xq, x_scale, counts, gate_q, gate_scale, up_q, up_scale, keep_i
     return act, inter13
 
 
+def _quantize_rows(x):
+    """x [N, D] bf16 -> (E4M3 codes uint8 [N, D], fp32 scale [N]) with the FP8 dispatch quantiser."""
+    lib = _lib.load()
+    N, D = x.shape
+    q = torch.empty((N, D), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((N,), dtype=torch.float32, device=x.device)
+    _lib.check(
+        lib.picomoe_fp8_quant(_lib.ptr(x), _lib.dtype_code(x.dtype), N, D, _lib.ptr(q), _lib.ptr(scale), _lib.stream_ptr()),
+        "picomoe_fp8_quant",
+    )
+    return q, scale
+
+
+def _down_fp8(act, counts, down_q, down_scale, row_weight):
+    """down GEMM on FP8 MFMA: the SwiGLU output ``act`` [N, I] bf16 is quantised per row here (one more pass over it),
+    ``down_q [E, H, I]`` / ``down_scale [E * H]`` as ``quantize_expert_weights(down_w)``."""
+    lib = _lib.load()
+    E, H, I = down_q.shape
+    N = act.shape[0]
+    aq, a_scale = _quantize_rows(act)
+    y = torch.empty((N, H), dtype=act.dtype, device=act.device)
+    _lib.check(
+        lib.picomoe_ffn_down_fp8(_lib.ptr(aq), _lib.ptr(a_scale), _lib.ptr(counts), E, N, H, I, _lib.ptr(down_q),
+                                 _lib.ptr(down_scale), _lib.ptr(row_weight), _lib.ptr(y), _lib.stream_ptr()),
+        "picomoe_ffn_down_fp8",
+    )
+    return y
+
+
 _workspaces = collections.OrderedDict()
 _MAX_WORKSPACES = 4
 
@@ -238,15 +267,17 @@ class _FusedMoE(torch.autograd.Function):
             return torch.empty((0, x.shape[1]), device=x.device, dtype=x.dtype)
         ctx.empty = False
         needs_grad = any(ctx.needs_input_grad[:4]) or (ctx.has_rw and ctx.needs_input_grad[5])
+        down_fp8 = None
         if fp8 is not None:
             # forward gate/up on FP8 MFMA from the dispatch's codes; the backward below is the bf16 one on x_sorted
-            xq, x_scale, gate_q, gate_scale, up_q, up_scale = fp8
+            xq, x_scale, gate_q, gate_scale, up_q, up_scale = fp8[:6]
+            down_fp8 = fp8[6:8] if len(fp8) >= 8 else None
             act, inter13 = _gate_up_fp8(xq.contiguous(), x_scale.contiguous(), counts, gate_q, gate_scale, up_q, up_scale,
                                         keep_inter13=needs_grad, dtype=x.dtype)
         else:
             act, inter13 = _gate_up(x, counts, gw, uw, keep_inter13=needs_grad)
         rw = row_weight.to(x.dtype).contiguous() if ctx.has_rw else None
-        y = _down(act, counts, dw, rw)
+        y = _down_fp8(act, counts, down_fp8[0], down_fp8[1], rw) if down_fp8 is not None else _down(act, counts, dw, rw)
         if needs_grad:
             ctx.save_for_backward(x, gw, uw, dw, act, inter13, rw)
         return y
@@ -286,8 +317,9 @@ def fused_moe(x_sorted, counts, gate_w, up_w, down_w, row_weight=None, fp8=None)
     """Differentiable fused MoE expert FFN.  counts [E] = per-expert row counts.
 
     ``fp8`` (optional, not in the reference): ``(xq [N,H] E4M3 codes, x_scale [N], gate_q, gate_scale, up_q,
-    up_scale)`` -- the rows of ``x_sorted`` as the FP8 dispatch ships them and the weights from
-    ``quantize_expert_weights``; the forward gate/up GEMM then runs on FP8 MFMA, everything else as without it."""
+    up_scale[, down_q, down_scale])`` -- the rows of ``x_sorted`` as the FP8 dispatch ships them and the weights from
+    ``quantize_expert_weights``; the forward gate/up GEMM then runs on FP8 MFMA and, when the down weights are given
+    too, so does the forward down GEMM (on the SwiGLU output quantised per row); the backward stays bf16."""
     return _FusedMoE.apply(x_sorted, gate_w, up_w, down_w, counts, row_weight, fp8)
 
 

@@ -49,10 +49,34 @@ def test_quant_full_benchmark_shape_bit_exact(gpu):
     assert q.element_size() * q.shape[1] + s.element_size() == 4100
 
 
-@pytest.mark.parametrize("hidden", [8, 40, 256, 1000, 2048, 4104, 8192, 16384])
+@pytest.mark.parametrize("hidden", [8, 40, 256, 1000, 2048, 4104, 8192, 8200, 14336, 16384, 16392, 32768, 32776])
 def test_quant_row_widths_bf16(gpu, hidden):
+    """Every kernel of the quantiser: a wave per row up to 8192 values (with and without a partly filled last chunk
+    round), a block per row up to 32768 (FFN 14336: the SwiGLU output of the FP8 down GEMM), the generic one beyond."""
     x = _c2_input(67, hidden, seed=hidden).bfloat16()
     _check(x, gpu)
+
+
+def test_quant_long_rows_edge_cases(gpu):
+    """Block-per-row kernel: a zero row (amax floor), a NaN, an inf, a huge finite value and the row maximum in the
+    last chunk."""
+    x = _c2_input(8, 14336, seed=3).bfloat16()
+    x[0] = 0
+    x[1, 14335] = float("nan")
+    x[2, 9000] = float("inf")
+    x[3, 14335] = 3.0e38
+    x[4, 14335] = 1000.0
+    x[5, 0] = -1000.0
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    q, s = C._per_token_quant_fp8(x.to(gpu))
+    q_ref, s_ref = O.quant_fp8(x)
+    qc = q.view(torch.uint8).cpu()
+    for r in (0, 3, 4, 5, 6, 7):
+        assert torch.equal(qc[r], q_ref[r]) and s[r].item() == s_ref[r].item(), r
+    # NaN / inf rows: the scale is NaN / inf as in the reference; codes of a NaN row are 0x7F by this build's convention
+    assert torch.isnan(s[1]).item() and torch.all((qc[1] & 0x7F) == 0x7F)
+    assert torch.isinf(s[2]).item()
 
 
 def test_quant_edge_rows_bf16(gpu):
