@@ -32,9 +32,43 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# L2 <-> memory bytes of the grouped-GEMM launches of one layer step, from two rocprofv3 --pmc runs of this script
-# (FETCH_SIZE x 2 KiB, WRITE_SIZE x 1 KiB; factors from the --traffic-probe copy kernel).  Algorithmic: 15.5e9.
-MEASURED_TRAFFIC_BYTES = {"c5": 35.2e9, "c2": 201.6e6}  # c2: the quantise kernel alone (algorithmic 201.4e6)
+# L2 <-> memory bytes per step (c5: the grouped-GEMM launches of one layer step; c2: the quantise kernel alone), from
+# two rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE; scale factors from the --traffic-probe copy kernel).
+# A counter run cannot happen inside a timed run, so the figure is carried here together with the digest of the kernel
+# sources it was measured on: `traffic` is reported only while the sources are still those, otherwise it is null.
+MEASURED_TRAFFIC = {
+    "c5": {"bytes": 35.2e9, "algorithmic_bytes": 15.5e9, "sources": "23e54c27ae92816f",
+           "files": ("ffn_mfma.hip", "mfma_tiles.h", "ffn.h", "common.h"),
+           "summary": "profiles/ffn_mfma_kernel_mixtral_hbm_traffic.txt"},
+    "c2": {"bytes": 201.6e6, "algorithmic_bytes": 201.4e6, "sources": "7103605a56574167",
+           "files": ("fp8_quant.hip", "common.h"),
+           "summary": "profiles/quant_bf16_wave_per_row_fp8_round_trip.txt"},
+}
+
+
+def kernel_sources_digest(files):
+    """sha256 over the named HIP kernel sources (names and contents, in name order), first 16 hex digits."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(files):
+        h.update(name.encode())
+        with open(os.path.join(ROOT, "picotron_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """(bytes or None, provenance dict) for the `roofline.traffic` field."""
+    m = MEASURED_TRAFFIC.get(workload)
+    if m is None:
+        return None, None
+    digest = kernel_sources_digest(m["files"])
+    current = m["sources"] == digest
+    return (m["bytes"] if current else None), {
+        "summary": m["summary"], "measured_on_sources": m["sources"], "this_build": digest, "current": current,
+        "algorithmic_bytes": m["algorithmic_bytes"]}
+
 
 WORKLOADS = {
     # name: tokens, hidden, ffn, experts, top_k, shared, capacity_factor, fp8_dispatch, backward
@@ -387,7 +421,8 @@ def fp8_bench(args):
         "config": {"workload": "FP8 round trip: 16384 x 4096 bf16 -> e4m3 + fp32 row scale -> bf16, 0.1 % outliers",
                    "rows": n, "hidden": h, "bytes_per_pass": pass_bytes, "round_trip_rel_l2": rel},
         "roofline": {"bound": "hbm", "achieved": pass_bytes / tq / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": pass_bytes / tq / 1e6 / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
+                     "frac": pass_bytes / tq / 1e6 / HBM_PEAK_GBPS, "traffic": measured_traffic("c2")[0],
+                     "traffic_source": measured_traffic("c2")[1],
                      "kernel": "quant_bf16_wave_per_row", "us": tq * 1e3,
                      "dequant": {"kernel": "dequant_bf16_wave_per_row", "achieved": pass_bytes / td / 1e6,
                                  "frac": pass_bytes / td / 1e6 / HBM_PEAK_GBPS, "us": td * 1e3}},
@@ -570,7 +605,8 @@ def main():
         achieved = total_flop / total_ms / 1e9  # TFLOP/s
         result["roofline"] = {
             "bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic(args.workload)[0],
+            "traffic_source": measured_traffic(args.workload)[1],
             "kernel": "ffn_mfma_kernel (grouped SwiGLU GEMMs: %s)" % ", ".join(kt),
             "flop_per_step": total_flop, "gemm_ms_per_step": total_ms,
             "launches": {k: {"ms": t, "tflops": f / t / 1e9} for k, (t, f) in kt.items()},

@@ -690,9 +690,12 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     }
 }
 
-// Second pass of a split last round: block b adds up the fp32 pieces of remainder tile b / 8 of XCD b % 8 (in piece
-// order, so the result does not depend on timing) and applies the epilogue of the unsplit kernel: accumulators rounded to
-// the output type; down: times the row weight, rounded again.
+// Second pass of a split last round: the blocks (b, y) add up the fp32 pieces of remainder tile b / 8 of XCD b % 8 (in
+// piece order, so the result does not depend on timing) and apply the epilogue of the unsplit kernel: accumulators
+// rounded to the output type; down: times the row weight, rounded again.  Block (b, y) takes rows 32y .. 32y + 31 of the
+// tile, eight per wavefront, and issues the loads of all its rows and pieces before it adds: one block per tile walking
+// its 256 rows took 20-75 us, the time of a load's latency per row.
+constexpr int kFixupRows = 32;
 template <int MODE>
 __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
     const GroupedLayout g = grouped_layout(p.counts, p.E, p.n_tiles, p.max_pieces);
@@ -703,11 +706,24 @@ __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
     const float* w = p.ws + (int64_t)(xcd * kCusPerXcd + t * g.pieces) * (BM * BN);
     const int c4 = (threadIdx.x & 63) * 4;
     if ((int64_t)tc.n_tile * BN + c4 >= p.N) return;  // columns past the output's last (N is a multiple of 8)
-    for (int row = threadIdx.x >> 6; row < tc.rows; row += 4) {
+    constexpr int kRowsPerWave = kFixupRows / 4;
+    const int row0 = blockIdx.y * kFixupRows + (threadIdx.x >> 6) * kRowsPerWave;
+    f32x4_t v[kRowsPerWave][kMaxSplit];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+        for (int pc = 0; pc < kMaxSplit; ++pc) {
+            const bool live = row0 + r < tc.rows && pc < g.pieces;
+            v[r][pc] = live ? *(const f32x4_t*)(w + (int64_t)pc * (BM * BN) + (row0 + r) * BN + c4) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        const int row = row0 + r;
+        if (row >= tc.rows) break;
         float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-        for (int pc = 0; pc < g.pieces; ++pc) {
-            const f32x4_t v = *(const f32x4_t*)(w + (int64_t)pc * (BM * BN) + row * BN + c4);
-            s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+#pragma unroll
+        for (int pc = 0; pc < kMaxSplit; ++pc) {  // pieces past g.pieces hold zeros: x + 0 leaves every sum as it is
+            s0 += v[r][pc][0]; s1 += v[r][pc][1]; s2 += v[r][pc][2]; s3 += v[r][pc][3];
         }
         s0 = bf16_bits_to_f32(f32_to_bf16_bits(s0)); s1 = bf16_bits_to_f32(f32_to_bf16_bits(s1));
         s2 = bf16_bits_to_f32(f32_to_bf16_bits(s2)); s3 = bf16_bits_to_f32(f32_to_bf16_bits(s3));
@@ -768,7 +784,7 @@ int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const 
     p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK);
     hipLaunchKernelGGL((ffn_mfma_kernel<kDown, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
     if (p.max_pieces > 1)
-        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDown>), dim3(kNumXcd * (kCusPerXcd / 2)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDown>), dim3(kNumXcd * (kCusPerXcd / 2), BM / kFixupRows), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -793,7 +809,7 @@ int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_
     p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK);
     hipLaunchKernelGGL((ffn_mfma_kernel<kDgradX, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
     if (p.max_pieces > 1)
-        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDgradX>), dim3(kNumXcd * (kCusPerXcd / 2)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDgradX>), dim3(kNumXcd * (kCusPerXcd / 2), BM / kFixupRows), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
