@@ -2,10 +2,15 @@
 // segments, forward + dgrad + wgrad, with the SwiGLU forward / backward fused into the epilogues.
 //
 // Block tile 256 x 256 x 64 (M x N x K), 8 wavefronts (two per SIMD), each owning a 128 x 64
-// sub-tile as 4 x 2 v_mfma_f32_32x32x16_bf16 accumulators (128 fp32 per lane).  Operand
+// sub-tile as 8 x 4 v_mfma_f32_16x16x32_bf16 accumulators (128 fp32 per lane).  The 16 x 16 x 32 shape is a matter of
+// power: an MFMA-only loop on random operands, where the chip's clock is set by the power it draws, runs 13-14 % faster
+// with it than with 32 x 32 x 16 (1788 against 1577 and 2020 against 1773 TFLOP/s on two boxes; both reach 2460 on
+// zeros) -- it reads and writes each accumulator once per 32 k values instead of once per 16.  (wgrad keeps
+// 4 x 2 accumulators of 32 x 32 x 16: its loop waits for its strided operand loads, and the higher clock the narrow
+// shape earns it only makes that wait longer in cycles -- 5 % slower in the layer.)  Operand
 // tiles go HBM/L2 -> LDS with 16-byte direct-to-LDS loads (no staging registers), two LDS stages of
 // 64 KB.  The k-loop is a ping-pong: the two waves of a SIMD alternate between a memory phase (fragment
-// reads) and an MFMA phase (8 MFMAs with the operand loads of the next k-tile and the L2 prefetch issued
+// reads) and an MFMA phase (16 MFMAs with the operand loads of the next k-tile and the L2 prefetch issued
 // between them), one phase apart.
 //
 // Two LDS tile layouts, chosen per operand by how it lies in memory:
@@ -67,8 +72,15 @@ struct MfmaParams {
     int max_pieces;       // 1 = no split
 };
 
-// X-major tiles: 16-byte chunk swizzle of k row kr (keeps the 8 rows one transpose read touches apart)
-__device__ __forceinline__ int swz_x(int kr) { return 4 * (kr & 3) + 16 * ((kr >> 3) & 1); }
+// X-major tiles: 16-byte chunk swizzle of k row kr.  One transpose read takes 32 bytes from each of 16 k rows (rows
+// 8g + j, g = 0..3, j = 0..3, plus a multiple of 4); rows are 512 B apart, i.e. on the same banks, and the swizzle puts the
+// eight rows the first half of the lanes addresses (g = 0, 1) on the eight 32-byte slots of the 256 bytes of banks.
+// With 32 x 32 MFMA blocks (wgrad) a read takes 64 bytes from each of 8 k rows (rows 8h + j, h = 0, 1), which the
+// swizzle spreads over the four 64-byte slots twice.
+template <bool WIDE>
+__device__ __forceinline__ int swz_x(int kr) {
+    return WIDE ? 4 * (kr & 3) + 16 * ((kr >> 3) & 1) : 2 * (kr & 3) + 8 * ((kr >> 3) & 1);
+}
 
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(8))) short s16x8_t;
@@ -112,10 +124,12 @@ __device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m
 template <int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     using T = Traits<MODE>;
-    constexpr int NI = 4;               // 32-row blocks per wave
-    constexpr int NJ = 16 / NW;         // 32-column blocks per wave (4 or 2)
+    constexpr bool kWide = MODE == kWgrad;  // 32 x 32 x 16 MFMA blocks instead of 16 x 16 x 32
+    constexpr int NI = 8;               // 16-row blocks per wave
+    constexpr int NJ = 4;               // 16-column blocks per wave
+    constexpr int WI = 4, WJ = 2;       // the same in 32 x 32 blocks
     constexpr int kWaveCols = NW / 2;   // wave grid: 2 rows x kWaveCols columns
-    constexpr int CW = NJ * 32;         // columns per wave
+    constexpr int CW = NJ * 16;         // columns per wave
     constexpr int QN = 32 / NW;         // direct-to-LDS load instructions per operand, wave and k-tile
     constexpr int RPW = QN * 8;         // K-major tile rows a wave fills
     constexpr int KPW = QN * 2;         // X-major k rows a wave fills
@@ -131,7 +145,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS bases and row ranges stay scalar
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
-    const int l31 = lane & 31, hi = lane >> 5;
+    const int l15 = lane & 15, g4 = lane >> 4;
     // k-tiles of this block: all of K, or this piece's share of it
     const int n_kt_all = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
     const int kt_first = kCanSplit ? (int)((int64_t)tc.piece * n_kt_all / tc.pieces) : 0;
@@ -170,7 +184,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
             const int kr = wave * KPW + q * 2 + (lane >> 5);
-            const int chunk = (lane & 31) ^ swz_x(kr);
+            const int chunk = (lane & 31) ^ swz_x<kWide>(kr);
             int64_t col = (int64_t)tc.m_tile * BM + chunk * 8;
             col = col + 8 <= p.M ? col : p.M - 8;
             a_off[q] = (uint32_t)(kr * (int)p.lda * 2 + (int)col * 2);
@@ -219,7 +233,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
             const int kr = wave * KPW + q * 2 + (lane >> 5);
-            const int chunk = (lane & 31) ^ swz_x(kr);
+            const int chunk = (lane & 31) ^ swz_x<kWide>(kr);
             int64_t col = (int64_t)tc.n_tile * BN + chunk * 8;
             col = col + 8 <= p.N ? col : p.N - 8;
             b_off[q] = (uint32_t)(kr * (int)p.ldb * 2 + (int)col * 2);
@@ -338,82 +352,134 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     // ------------------------------------------------------------------------------------------
     // LDS -> fragments
     // ------------------------------------------------------------------------------------------
-    // K-major: lane reads row (l & 31) of a 32-row block, 16-byte k chunk (2*kk + (l >> 5)).
-    // X-major: two transpose reads per fragment; lane addresses 8 bytes of k row 16kk + 8*(l>>5) + 4t + ((l>>2)&3)
-    //          at column 16*((l>>4)&1) + 4*(l&3) of the 32-column block and receives k rows 16kk + 8*(l>>5) + 4t..+3
-    //          of column 16*((l>>4)&1) + (l&15).
-    // One address register per fragment block, pointing at k sub-step 0 of the current stage.  K-major: the
-    // swizzle XORs the chunk index, and (2kk + hi) ^ f == (hi ^ f) ^ 2kk, so sub-step kk is that address XOR
-    // (kk << 5) -- one VALU op at the use; X-major: the sub-step is an immediate offset.  One XOR per register
-    // and k-tile flips between the two stages.
-    uint32_t a_ad[NI], b_ad[NJ];
+    // An MFMA takes 32 k values: a k-tile is two sub-steps.  Operand lane l holds row / column (l & 15) of a 16-wide block
+    // and the 8 k values 8*(l >> 4) .. +7 of the sub-step.
+    // K-major: lane reads row (l & 15) of a 16-row block, 16-byte k chunk 4*sub + (l >> 4).  The swizzle XORs the chunk
+    //          index and depends on (row >> 1) & 7 only, which is the same in every 16-row block: one address register
+    //          per operand, block b at + b * 2048 (an immediate), sub-step sub at XOR (sub << 6).
+    // X-major: two transpose reads per fragment; lane addresses 8 bytes of k row 32*sub + 8*(l>>4) + 4t + ((l>>2)&3) at
+    //          column 4*(l&3) of the 16-column block and receives k rows 32*sub + 8*(l>>4) + 4t..+3 of column (l & 15).
+    //          sub and t are immediates (whole k rows), block b is XOR (b << 5): the block index sits in bits of the chunk
+    //          index that the swizzle also flips, and XOR commutes where + does not.
+    // One XOR per register and k-tile flips between the two stages.
+    uint32_t a_ad, b_ad;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-    const int xg = 4 * ((lane >> 2) & 3) + 16 * hi;  // swz_x of the k row this lane addresses
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
+    {
+        const int kr = 8 * g4 + ((lane >> 2) & 3);  // X-major: the k row this lane addresses (sub-step 0, t = 0)
+        const int h = (lane & 3) >> 1;              // which 16-byte chunk of the block's 32 bytes
+        const int in_chunk = (4 * (lane & 1)) << 1; // byte offset of the lane's 4 columns inside the chunk
         if (T::kAKMajor) {
-            const int ra = wm * 128 + i * 32 + l31;
-            a_ad[i] = lds0 + ra * 128 + ((hi ^ swz(ra)) << 4);
+            const int ra = wm * 128 + l15;
+            a_ad = lds0 + ra * 128 + ((g4 ^ swz(ra)) << 4);
         } else {
-            const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            a_ad[i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            a_ad = lds0 + kr * 512 + (((wm * 16 + h) ^ swz_x<kWide>(kr)) << 4) + in_chunk;
+        }
+        if (T::kBKMajor) {
+            const int rb = wn * CW + l15;
+            b_ad = lds0 + kTileBytes + rb * 128 + ((g4 ^ swz(rb)) << 4);
+        } else {
+            b_ad = lds0 + kTileBytes + kr * 512 + (((wn * 8 + h) ^ swz_x<kWide>(kr)) << 4) + in_chunk;
         }
     }
+    // 32 x 32 blocks (wgrad, both operands X-major): one address register per block; lane addresses 8 bytes of k row
+    // 16kk + 8*(l>>5) + 4t + ((l>>2)&3) at column 16*((l>>4)&1) + 4*(l&3) of the 32-column block and receives k rows
+    // 16kk + 8*(l>>5) + 4t..+3 of column 16*((l>>4)&1) + (l&15).
+    uint32_t a_adw[WI], b_adw[WJ];
+    if (kWide) {
+        const int hi = lane >> 5;
+        const int xg = swz_x<true>(8 * hi + ((lane >> 2) & 3));
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        if (T::kBKMajor) {
-            const int rb = wn * CW + j * 32 + l31;
-            b_ad[j] = lds0 + kTileBytes + rb * 128 + ((hi ^ swz(rb)) << 4);
-        } else {
+        for (int i = 0; i < WI; ++i) {
+            const int col = wm * 128 + i * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            a_adw[i] = lds0 + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+        }
+#pragma unroll
+        for (int j = 0; j < WJ; ++j) {
             const int col = wn * CW + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            b_ad[j] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
+            b_adw[j] = lds0 + kTileBytes + (((col >> 3) ^ xg) << 4) + ((col & 7) << 1) + (8 * hi + ((lane >> 2) & 3)) * 512;
         }
     }
     auto flip_stage = [&]() {
+        if (kWide) {
 #pragma unroll
-        for (int i = 0; i < NI; ++i) a_ad[i] ^= (uint32_t)kStageBytes;
+            for (int i = 0; i < WI; ++i) a_adw[i] ^= (uint32_t)kStageBytes;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) b_ad[j] ^= (uint32_t)kStageBytes;
+            for (int j = 0; j < WJ; ++j) b_adw[j] ^= (uint32_t)kStageBytes;
+        } else {
+            a_ad ^= (uint32_t)kStageBytes;
+            b_ad ^= (uint32_t)kStageBytes;
+        }
     };
 
-    f32x16_t acc[NI][NJ];
+    f32x4_t acc[NI][NJ];     // 16 x 16 blocks
+    f32x16_t accw[WI][WJ];   // 32 x 32 blocks (wgrad); only the set the kernel uses exists in the compiled code
+    if (kWide) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+        for (int i = 0; i < WI; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+            for (int j = 0; j < WJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+                for (int r = 0; r < 16; ++r) accw[i][j][r] = 0.f;
+    } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+    }
 
-    bf16x8_t af[NI], bfr[NJ];
-    auto read_tr_frag = [&](uint32_t ad, int kk) -> bf16x8_t {
-        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512)));
-        const s16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + kk * (16 * 512) + 4 * 512));
+    // The 32 MFMAs of a sub-step are two phases of 16: rows 0..63 of the wave's 128 (blocks 0..3), then rows 64..127.
+    // A phase holds its four A fragments and the sub-step's four B fragments, which the first phase of a sub-step reads.
+    bf16x8_t af[4], bfr[NJ];
+    auto read_b128 = [&](uint32_t ad) -> bf16x8_t { return *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)ad; };
+    auto read_tr_frag = [&](uint32_t ad) -> bf16x8_t {
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)ad);
+        const s16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(ad + 4 * 512));
         const s16x8_t v = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
         return __builtin_bit_cast(bf16x8_t, v);
     };
-    // reads the fragments of k sub-step kk from the stage the address registers currently point at
+    auto read_a = [&](int ib, int sub) -> bf16x8_t {
+        if (T::kAKMajor) return read_b128((a_ad ^ (uint32_t)(sub << 6)) + ib * 2048);
+        return read_tr_frag((a_ad ^ (uint32_t)(ib << 5)) + sub * (32 * 512));
+    };
+    auto read_b = [&](int jb, int sub) -> bf16x8_t {
+        if (T::kBKMajor) return read_b128((b_ad ^ (uint32_t)(sub << 6)) + jb * 2048);
+        return read_tr_frag((b_ad ^ (uint32_t)(jb << 5)) + sub * (32 * 512));
+    };
+    // 16-row blocks of phase kk (sub-step kk >> 1, half kk & 1) that hold rows of the segment, given the wave's live
+    // 32-row blocks
+    auto live_blocks = [](int kk, int active32) {
+        const int n = 2 * active32 - 4 * (kk & 1);
+        return n < 0 ? 0 : (n > 4 ? 4 : n);
+    };
+    // reads the fragments of phase kk from the stage the address registers currently point at
+    // (wide blocks: phase kk is the sub-step of 16 k values kk, 4 A and 2 B fragments, two transpose reads each)
+    auto read_wide = [&](uint32_t ad, int kk) -> bf16x8_t { return read_tr_frag(ad + kk * (16 * 512)); };
     auto read_frags = [&](int kk, auto active) {
-        constexpr int kActiveBlocks = decltype(active)::value;
-        if (kActiveBlocks == 0) return;
+        constexpr int kActive32 = decltype(active)::value;
+        if (kActive32 == 0) return;
+        if (kWide) {
 #pragma unroll
-        for (int i = 0; i < kActiveBlocks; ++i) {
-            if (T::kAKMajor)
-                af[i] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(a_ad[i] ^ (uint32_t)(kk << 5));
-            else
-                af[i] = read_tr_frag(a_ad[i], kk);
+            for (int i = 0; i < kActive32; ++i) af[i] = read_wide(a_adw[i], kk);
+#pragma unroll
+            for (int j = 0; j < WJ; ++j) bfr[j] = read_wide(b_adw[j], kk);
+            return;
         }
+        const int sub = kk >> 1, half = kk & 1;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            if (T::kBKMajor)
-                bfr[j] = *(__attribute__((address_space(3))) const bf16x8_t*)(uintptr_t)(b_ad[j] ^ (uint32_t)(kk << 5));
-            else
-                bfr[j] = read_tr_frag(b_ad[j], kk);
+        for (int i = 0; i < 4; ++i)
+            if (i < live_blocks(kk, kActive32)) af[i] = read_a(4 * half + i, sub);
+        if (half == 0) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bfr[j] = read_b(j, sub);
         }
     };
     // wgrad, last k-tile: zero the fragment elements whose k row lies past the expert's last row
     auto mask_tail = [&](int kt, int kk) {
         if (MODE != kWgrad) return;
-        const int valid = tc.rows - kt * BK - kk * 16 - 8 * hi;  // lane holds k = 8*hi + 0..7 of this sub-step
+        // lane holds k = 8*(l >> 4) + 0..7 of its sub-step of 32 (wide blocks: 8*(l >> 5) + 0..7 of its sub-step of 16)
+        const int valid = kWide ? tc.rows - kt * BK - kk * 16 - 8 * (lane >> 5) : tc.rows - kt * BK - (kk >> 1) * 32 - 8 * g4;
         if (valid >= 8) return;
         auto zero_tail = [&](bf16x8_t& f) {
             s16x8_t a = __builtin_bit_cast(s16x8_t, f);
@@ -423,19 +489,35 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             f = __builtin_bit_cast(bf16x8_t, a);
         };
 #pragma unroll
-        for (int i = 0; i < NI; ++i) zero_tail(af[i]);
+        for (int i = 0; i < 4; ++i) zero_tail(af[i]);
+        if (kWide || (kk & 1) == 0) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) zero_tail(bfr[j]);
+            for (int j = 0; j < (kWide ? WJ : NJ); ++j) zero_tail(bfr[j]);
+        }
     };
-    // The MFMAs of one k-sub-step with side(n) run after MFMA n (n = 0 .. NI*NJ - 1): the slots for this wave's loads.
+    // The 16 MFMAs of phase kk with side(n) run after MFMA n (n = 0 .. 15): the slots for this wave's loads.
     // `active` carries the number of 32-row blocks the wave computes; a wave without rows runs the side jobs alone.
-    auto mma_with = [&](auto active, auto side) {
+    auto mma_with = [&](int kk, auto active, auto side) {
+        if (kWide) {  // 8 MFMAs of 32 x 32 x 16, side(n) after MFMA n (n = 0 .. 7)
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
+            for (int i = 0; i < WI; ++i)
+#pragma unroll
+                for (int j = 0; j < WJ; ++j) {
+                    if (i < decltype(active)::value)
+                        accw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], accw[i][j], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    side(i * WJ + j);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            return;
+        }
+        const int half = kk & 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                if (i < decltype(active)::value)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+                if (i < live_blocks(kk, decltype(active)::value))
+                    acc[4 * half + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[4 * half + i][j], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 side(i * NJ + j);
                 __builtin_amdgcn_sched_barrier(0);
@@ -456,15 +538,16 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         __syncthreads();
     }
     // The k-loop, a ping-pong between two groups of waves.  The eight waves form two groups, one wave of every SIMD in
-    // each (waves 0-3 own tile rows 0..127, waves 4-7 rows 128..255).  A k-sub-step (16 of the 64 k values) is a memory
-    // phase -- the LDS reads of its fragments, in sub-step 3 also the wait for the next k-tile -- followed by an MFMA phase:
-    // its 8 MFMAs, and between them this wave's direct-to-LDS loads of the next k-tile (sub-steps 0 and 1, one load after
-    // every second MFMA) and the L2 prefetch (sub-step 2).  Every phase ends in a barrier and the second group runs one
+    // each (waves 0-3 own tile rows 0..127, waves 4-7 rows 128..255).  A k-step is four pairs of phases (two sub-steps of
+    // 32 k values, each in two halves of the wave's rows).  A pair is a memory phase -- the LDS reads of its fragments, in
+    // the fourth also the wait for the next k-tile -- followed by an MFMA phase: its 16 MFMAs, and between them this
+    // wave's direct-to-LDS loads of the next k-tile (pairs 0 and 1, one load after every fourth MFMA) and the L2 prefetch
+    // (pair 2).  Every phase ends in a barrier and the second group runs one
     // phase behind the first, so while one wave of a SIMD reads LDS the other owns the MFMA pipe.
     // Where the loads sit matters.  A vector memory instruction holds its wave for some tens of cycles at issue.  In the
     // memory phase that time adds to the LDS reads, which alone take about as long as the other group's MFMAs (measured
     // with a cycle counter at every barrier: memory phases with loads ran 440-470 ticks against 341 for 8 MFMAs, the
-    // ones without 364-400); between two MFMAs it is free, the matrix pipe being busy for 32 cycles per MFMA anyway.
+    // ones without 364-400); between two MFMAs it is free, the matrix pipe being busy anyway (16 cycles per MFMA).
     // (History of the loop, each step measured side by side in one run: reads, loads and MFMAs interleaved finely in one
     // stream with two free-running waves per SIMD -- the older wave wins every MFMA slot and then idles a third of the
     // time at the k-step barrier; ping-pong with the loads in the memory phases, +8 %; loads in the MFMA phases, +4-7 %.)
@@ -504,13 +587,16 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 if (tail) mask_tail(kt, kk);
                 phase_end();
                 // MFMA phase
-                mma_with(active, [&](int n) {
-                    if (kk < 2 && (n & 1) == 0) {
-                        const int q = (QN / 2) * kk + (n >> 2);  // n = 0, 2: loads q of A and B; n = 4, 6: loads q + 1
-                        if ((n & 2) == 0) issue_a_at(a_next, next_is_last, stage ^ 1, q);
+                // load slots: every fourth of the 16 MFMAs (wide blocks: every second of the 8): one per 64 MFMA cycles
+                constexpr int kSlotShift = kWide ? 1 : 2;
+                mma_with(kk, active, [&](int n) {
+                    if (kk < 2 && (n & ((1 << kSlotShift) - 1)) == 0) {
+                        const int m = n >> kSlotShift;             // 0 .. 3
+                        const int q = (QN / 2) * kk + (m >> 1);    // m = 0, 1: loads q of A and B; m = 2, 3: loads q + 1
+                        if ((m & 1) == 0) issue_a_at(a_next, next_is_last, stage ^ 1, q);
                         else issue_b_at(b_next, next_is_last, stage ^ 1, q);
                     }
-                    if (kk == 2 && n == 1) prefetch_l2(kt);
+                    if (kk == 2 && n == (kWide ? 1 : 2)) prefetch_l2(kt);
                 });
                 if (kk == 3) {
                     flip_stage();
@@ -550,10 +636,10 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     __syncthreads();
 
     // ------------------------------------------------------------------------------------------
-    // epilogue.  A lane holds column (l & 31) and rows 8*(r/4) + 4*(l >> 5) + (r % 4) of each 32 x 32
+    // epilogue.  A lane holds column (l & 15) and rows 4*(l >> 4) + r (r = 0..3) of each 16 x 16
     // accumulator block: consecutive lanes are consecutive columns, 2 bytes apart in the output.  Each wave
-    // therefore stages 32 rows at a time through its own slice of LDS (the operand stages are free after
-    // the last barrier) and reads them back row-contiguously, so HBM sees 16-byte lanes and 128..256-byte
+    // therefore stages 32 rows (two blocks) at a time through its own slice of LDS (the operand stages are free
+    // after the last barrier) and reads them back row-contiguously, so HBM sees 16-byte lanes and 128..256-byte
     // row segments, and the fused SwiGLU backward reads g / u the same way.
     // ------------------------------------------------------------------------------------------
     if (kCanSplit && tc.pieces > 1) {
@@ -565,9 +651,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-                    if (row < tc.rows) w[row * BN + wn * CW + j * 32 + l31] = acc[i][j][r];
+                for (int r = 0; r < 4; ++r) {
+                    const int row = wm * 128 + i * 16 + g4 * 4 + r;
+                    if (row < tc.rows) w[row * BN + wn * CW + j * 16 + l15] = acc[i][j][r];
                 }
         return;
     }
@@ -585,14 +671,29 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
     static_assert(kReadIters >= 1, "a pass must cover at least one chunk per lane");
 
-    auto stage_block = [&](auto value) {  // value(j, r) -> float, j over the 32-column blocks of this pass
+    // value(b, j, r) -> float: 16-row block b (0, 1) of the 32 rows, j over the 16-column blocks of this pass, register r
+    auto stage_block = [&](auto value) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // earlier read-backs of this slice are done
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int j = 0; j < kEpiCols / 16; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = b * 16 + g4 * 4 + r;
+                    *(uint16_t*)(epi + row * kEpiStride + (j * 16 + l15) * 2) = (uint16_t)f32_to_bf16_bits(value(b, j, r));
+                }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    // the same for a 32 x 32 block row: a lane holds column (l & 31) and rows 8*(r/4) + 4*(l >> 5) + (r % 4); value(j, r)
+    auto stage_block_wide = [&](auto value) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int j = 0; j < kEpiCols / 32; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
-                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + l31) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
+                const int row = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + (lane & 31)) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
             }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
@@ -608,19 +709,23 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     };
 
+    // i runs over the wave's four 32-row passes; pass i holds the accumulator blocks 2i and 2i + 1
     if (MODE == kGateUp) {
         const int64_t I = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < 4; ++i) {
             if (wm * 128 + i * 32 >= valid_rows) continue;  // wave-uniform: a block of rows past the segment has nothing to store
             // g and u rounded to bf16 in place (what the reference's two Linear outputs hold)
 #pragma unroll
-            for (int j = 0; j < NJ; ++j)
+            for (int b = 0; b < 2; ++b)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][r]));
-            stage_block([&](int j, int r) {
-                const float g = acc[i][j][r], u = acc[i][j + NJ / 2][r];
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[2 * i + b][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][j][r]));
+            // column blocks 0, 1 of the wave hold g, blocks 2, 3 the u of the same output columns
+            stage_block([&](int b, int j, int r) {
+                const float g = acc[2 * i + b][j][r], u = acc[2 * i + b][j + NJ / 2][r];
                 return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
             });
             // (I is a multiple of 8: a 16-byte chunk lies inside the row or past its end as a whole)
@@ -628,11 +733,11 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                 if (col0 + c < I) *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v;
             });
             if (p.out2) {
-                stage_block([&](int j, int r) { return acc[i][j][r]; });
+                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) {
                     if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v;
                 });
-                stage_block([&](int j, int r) { return acc[i][j + NJ / 2][r]; });
+                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j + NJ / 2][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) {
                     if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v;
                 });
@@ -641,9 +746,10 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     } else {
         const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < 4; ++i) {
             if (wm * 128 + i * 32 >= valid_rows) continue;
-            stage_block([&](int j, int r) { return acc[i][j][r]; });
+            if (kWide) stage_block_wide([&](int j, int r) { return accw[i][j][r]; });
+            else stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
             for_chunks(i, [&](int trow, int c, u32x4_t v) {
                 const int64_t col = col0 + c;
                 if (col >= p.N) return;
