@@ -279,7 +279,7 @@ def fp8_gemm_variant(moe, step, w, steps):
                 out = {"ms_per_step": ms, "tokens_per_s": w["T"] / (ms * 1e-3), "gate_up_fp8_ms": gu_ms,
                        "gate_up_fp8_tflops": gu_flop / gu_ms / 1e9, "frac_fp8_mfma_peak": gu_flop / gu_ms / 1e9 / 5000.0,
                        "weight_quant_ms_per_step": q_ms,
-                       "note": "forward gate/up on v_mfma_f32_32x32x64_f8f6f4; down, dgrad and wgrad stay bf16; not the headline value"}
+                       "note": "forward gate/up on v_mfma_f32_16x16x128_f8f6f4; down, dgrad and wgrad stay bf16; not the headline value"}
             else:
                 # _down_fp8 = the row quantiser of the SwiGLU output + the FP8 down kernel; the kernel alone is the difference
                 d_ms, aq_ms = per_call("_down_fp8"), per_call("_quantize_rows")

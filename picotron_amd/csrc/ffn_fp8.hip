@@ -1,14 +1,15 @@
 // FP8 (E4M3) MFMA kernels for the forward projections of the expert FFN on gfx950 (MI355X): per-row quantised
 // activations (codes + one fp32 scale per row: the FP8 dispatch's rows for gate/up, the quantised SwiGLU output for
-// down) meet expert weights quantised the same way (one scale per output row) in v_mfma_f32_32x32x64_f8f6f4, fp32
+// down) meet expert weights quantised the same way (one scale per output row) in v_mfma_f32_16x16x128_f8f6f4, fp32
 // accumulation, and the two scales are applied to the accumulators in the epilogue -- fused with SwiGLU for gate/up,
 // with the optional row weight for down.
 //
 // Same frame as the bf16 kernels: 256 x 256 block tile, 8 wavefronts (two per SIMD) of 128 x 64, two 64 KB LDS
-// stages filled by 16-byte direct-to-LDS loads.  A 128-byte LDS row now holds 128 k values, so one k-step is two
-// MFMA sub-steps of K = 64 and a tile needs half as many k-steps, loads and barriers per FLOP.  A lane feeds an MFMA
-// with 32 consecutive k bytes of its row (two ds_read_b128); which 32 of the 64 go to which lane half is free as
-// long as both operands agree, because the instruction only sums over k.
+// stages filled by 16-byte direct-to-LDS loads.  A 128-byte LDS row now holds 128 k values, which one MFMA consumes
+// whole: a tile needs half as many k-steps, loads and barriers per FLOP.  A lane feeds an MFMA with 32 consecutive k
+// bytes of its row (two ds_read_b128); which 32 of the 128 go to which lane group is free as long as both operands
+// agree, because the instruction only sums over k.  (16 x 16 x 128 rather than 32 x 32 x 64: under the power cap a loop of
+// nothing but MFMAs on random data runs 8 % faster with it.)
 #include <type_traits>
 
 #include "ffn.h"
@@ -43,7 +44,7 @@ struct Fp8Params {
 
 template <int MODE>
 __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p) {
-    constexpr int NI = 4, NJ = 2, kWaveCols = 4, CW = 64, QN = 4, RPW = 32;
+    constexpr int NI = 8, NJ = 4, kWaveCols = 4, CW = 64, QN = 4, RPW = 32;
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
     TileCoord tc;
     if (!locate_m_grouped(p.counts, p.E, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
@@ -51,7 +52,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
-    const int l31 = lane & 31, hi = lane >> 5;
+    const int l15 = lane & 15, g4 = lane >> 4;
     const int n_kt = (int)(p.K / kFp8BK);
     const bool wave_active = wm * 128 < tc.rows;
 
@@ -86,59 +87,51 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         }
     };
 
-    // LDS -> fragments.  Lane (row l & 31, half l >> 5) of sub-step s reads the 16-byte chunks 4s + 2*half and
-    // 4s + 2*half + 1 of its row; with the XOR swizzle those are the address of chunk 2*half XOR (s << 6) and XOR 16.
-    uint32_t a_ad[NI], b_ad[NJ];
+    // LDS -> fragments.  An MFMA takes all 128 k values of a row: lane (row l & 15 of a 16-row block, k group l >> 4)
+    // supplies the 32 bytes of k group l >> 4, the 16-byte chunks 2*(l >> 4) and 2*(l >> 4) + 1 of its row; with the XOR
+    // swizzle the second is the address of the first XOR 16.  The swizzle depends on (row >> 1) & 7 only, which is the
+    // same in every 16-row block: one address register per operand, block b at + b * 2048.
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int ra = wm * 128 + i * 32 + l31;
-        a_ad[i] = lds0 + ra * 128 + (((2 * hi) ^ swz(ra)) << 4);
-    }
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        const int rb = wn * CW + j * 32 + l31;
-        b_ad[j] = lds0 + kTileBytes + rb * 128 + (((2 * hi) ^ swz(rb)) << 4);
-    }
+    const int ra = wm * 128 + l15, rb = wn * CW + l15;
+    uint32_t a_ad = lds0 + ra * 128 + (((2 * g4) ^ swz(ra)) << 4);
+    uint32_t b_ad = lds0 + kTileBytes + rb * 128 + (((2 * g4) ^ swz(rb)) << 4);
     auto flip_stage = [&]() {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) a_ad[i] ^= (uint32_t)kStageBytes;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) b_ad[j] ^= (uint32_t)kStageBytes;
+        a_ad ^= (uint32_t)kStageBytes;
+        b_ad ^= (uint32_t)kStageBytes;
     };
-    auto read_frag = [&](uint32_t ad, int s) -> i32x8_t {
-        const u32x4_t lo = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)(ad ^ (uint32_t)(s << 6));
-        const u32x4_t up = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)(ad ^ (uint32_t)(s << 6) ^ 16u);
+    auto read_frag = [&](uint32_t ad) -> i32x8_t {
+        const u32x4_t lo = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)ad;
+        const u32x4_t up = *(__attribute__((address_space(3))) const u32x4_t*)(uintptr_t)(ad ^ 16u);
         i32x8_t v;
         v[0] = (int)lo[0]; v[1] = (int)lo[1]; v[2] = (int)lo[2]; v[3] = (int)lo[3];
         v[4] = (int)up[0]; v[5] = (int)up[1]; v[6] = (int)up[2]; v[7] = (int)up[3];
         return v;
     };
 
-    f32x16_t acc[NI][NJ];
+    f32x4_t acc[NI][NJ];
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    i32x8_t af[2][NI], bfr[2][NJ];
-    // fragment f of sub-step sub into buffer buf: f = 0..3 the A row blocks, 4..5 the B column blocks
-    auto read_one = [&](int f, int sub, int buf) {
-        if (f < NI) af[buf][f] = read_frag(a_ad[f], sub);
-        else bfr[buf][f - NI] = read_frag(b_ad[f - NI], sub);
-    };
-    // the 8 MFMAs (64 cycles each) of one sub-step with side(n) run after MFMA n: the slots for LDS reads and loads
-    auto mma_with = [&](int buf, auto active, auto side) {
+    // A k-step is two halves of 16 MFMAs: rows 0..63 of the wave's 128 (A blocks 0..3), then rows 64..127 (blocks 4..7),
+    // each against the four B blocks.  af[h] holds the four A fragments of half h, bfr the B fragments of the k-tile.
+    i32x8_t af[2][4], bfr[NJ];
+    auto read_a = [&](int h, int i) { af[h][i] = read_frag(a_ad + (4 * h + i) * 2048); };
+    auto read_b = [&](int j) { bfr[j] = read_frag(b_ad + j * 2048); };
+    // the 16 MFMAs (32 cycles each) of half h, B block by B block, with side(n) run after MFMA n: the slots for LDS
+    // reads and loads.  After MFMA 4j + 3 nothing in this k-step needs bfr[j] any more.
+    auto mma_with = [&](int h, auto active, auto side) {
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
+            for (int i = 0; i < 4; ++i) {
                 if (decltype(active)::value)
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[buf][i], bfr[buf][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                    acc[4 * h + i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[h][i], bfr[j], acc[4 * h + i][j], 0, 0, 0, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                side(i * NJ + j);
+                side(j * 4 + i);
                 __builtin_amdgcn_sched_barrier(0);
             }
     };
@@ -154,22 +147,24 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         __syncthreads();
         if (wave_active) {
 #pragma unroll
-            for (int f = 0; f < NI + NJ; ++f) read_one(f, 0, 0);
+            for (int i = 0; i < 4; ++i) read_a(0, i);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) read_b(j);
         }
     }
-    // One k-step = two sub-steps.  Sub-step 0: its MFMAs with the fragment reads of sub-step 1 between them; then every
-    // wave holds its last fragments of this stage in registers, waits for its loads of the next k-tile (issued a whole
-    // k-step ago) and meets the others at the barrier.  Sub-step 1: its MFMAs with all 8 loads of k-tile kt+2 into the
-    // stage just vacated, two after each of the first four MFMAs (issued right after the barrier they have the longest
-    // time to land: split 4 + 4 around the barrier the kernel was 4.5 % slower, one per MFMA 2 % slower), and the fragment
-    // reads of sub-step 0 of k-tile kt+1 from the other stage after MFMAs 2..7.
+    // One k-step.  First half: its MFMAs with the reads of the second half's A fragments between them; then every wave
+    // holds its last fragments of this stage in registers, waits for its loads of the next k-tile (issued a whole k-step
+    // ago) and meets the others at the barrier.  Second half: its MFMAs with all 8 loads of k-tile kt+2 into the stage just
+    // vacated, one after each of the first eight MFMAs (issued right after the barrier they have the longest time to
+    // land), and the fragment reads of k-tile kt+1 from the other stage: the first half's A fragments after MFMAs 8..11,
+    // B block j after MFMA 4j + 3, the last MFMA of the k-step that multiplies by the old one.
     auto k_loop = [&](auto active) {
         constexpr bool kActive = decltype(active)::value;
         for (int kt = 0; kt < n_kt; ++kt) {
             const int stage = kt & 1;
             const int kt_load = kt + 2 < n_kt ? kt + 2 : n_kt - 1;  // clamped past the end: lands in a dead stage
             mma_with(0, active, [&](int n) {
-                if (kActive && n < NI + NJ) read_one(n, 1, 1);
+                if (kActive && (n & 1) == 0 && n < 8) read_a(1, n >> 1);
             });
             __builtin_amdgcn_s_waitcnt(0x0F70);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -178,8 +173,13 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
             __builtin_amdgcn_sched_barrier(0);
             flip_stage();
             mma_with(1, active, [&](int n) {
-                if (n < 4) { issue_a(kt_load, stage, n); issue_b(kt_load, stage, n); }
-                if (kActive && n >= 2) read_one(n - 2, 0, 0);  // past the last tile this reads a stage that is not used any more
+                if (n < 8) {
+                    if ((n & 1) == 0) issue_a(kt_load, stage, n >> 1);
+                    else issue_b(kt_load, stage, n >> 1);
+                }
+                // past the last tile these read a stage that is not used any more
+                if (kActive && (n & 3) == 3) read_b(n >> 2);
+                if (kActive && n >= 8 && n < 12) read_a(0, n - 8);
             });
         }
     };
@@ -189,7 +189,8 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     __syncthreads();
 
     // epilogue: the two scales, rounding to bf16, and 32 rows at a time through a wave-private slice of LDS so that the
-    // stores are 16-byte lanes of contiguous rows
+    // stores are 16-byte lanes of contiguous rows.  A lane holds column (l & 15) and rows 4*(l >> 4) + r (r = 0..3) of
+    // each 16 x 16 accumulator block.
     float* row_scale = (float*)(lds + kStageBytes);  // 256 floats, past the staging slices
     if (tid < BM) row_scale[tid] = p.x_scale[tc.row0 + (tid < tc.rows ? tid : tc.rows - 1)];
     constexpr int kEpiCols = MODE == kFp8GateUp ? CW / 2 : CW;
@@ -197,15 +198,17 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     char* epi = lds + wave * (32 * kEpiStride);
     constexpr int kChunksPerRow = kEpiCols / 8;
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
-    auto stage_block = [&](auto value) {  // value(j, r), j over the 32-column blocks of a pass
+    auto stage_block = [&](auto value) {  // value(b, j, r): 16-row block b of the 32 rows, 16-column block j, row r of 4
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int j = 0; j < kEpiCols / 32; ++j)
+        for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = (r >> 2) * 8 + hi * 4 + (r & 3);
-                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + l31) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
-            }
+            for (int j = 0; j < kEpiCols / 16; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = b * 16 + g4 * 4 + r;
+                    *(uint16_t*)(epi + row * kEpiStride + (j * 16 + l15) * 2) = (uint16_t)f32_to_bf16_bits(value(b, j, r));
+                }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
     auto for_chunks = [&](int i, auto f) {
@@ -219,28 +222,39 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         }
     };
     if (MODE == kFp8GateUp) {
-        // g and u rounded to bf16 (what the two Linear outputs of the reference hold), then SwiGLU
+        // g and u rounded to bf16 (what the two Linear outputs of the reference hold), then SwiGLU.  B blocks 0, 1 of the
+        // wave are its 32 gate columns, blocks 2, 3 the up columns of the same FFN columns.
         const int64_t I = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
-        const float gs = p.g_scale[(int64_t)tc.e * I + col0 + l31], us = p.u_scale[(int64_t)tc.e * I + col0 + l31];
+        float gs[2], us[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            gs[j] = p.g_scale[(int64_t)tc.e * I + col0 + j * 16 + l15];
+            us[j] = p.u_scale[(int64_t)tc.e * I + col0 + j * 16 + l15];
+        }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < NI / 2; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float sx = row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)];
-                acc[i][0][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][r] * sx * gs));
-                acc[i][1][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][r] * sx * us));
-            }
-            stage_block([&](int, int r) {
-                const float g = acc[i][0][r], u = acc[i][1][r];
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float sx = row_scale[wm * 128 + i * 32 + b * 16 + g4 * 4 + r];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        acc[2 * i + b][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][j][r] * sx * gs[j]));
+                        acc[2 * i + b][2 + j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][2 + j][r] * sx * us[j]));
+                    }
+                }
+            stage_block([&](int b, int j, int r) {
+                const float g = acc[2 * i + b][j][r], u = acc[2 * i + b][2 + j][r];
                 return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
             });
             for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.act + (tc.row0 + trow) * I + col0 + c) = v; });
             if (p.inter13) {
-                stage_block([&](int, int r) { return acc[i][0][r]; });
+                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + col0 + c) = v; });
-                stage_block([&](int, int r) { return acc[i][1][r]; });
+                stage_block([&](int b, int j, int r) { return acc[2 * i + b][2 + j][r]; });
                 for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + I + col0 + c) = v; });
             }
         }
@@ -250,13 +264,13 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
         float ws[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) ws[j] = p.g_scale[(int64_t)tc.e * H + col0 + j * 32 + l31];
+        for (int j = 0; j < NJ; ++j) ws[j] = p.g_scale[(int64_t)tc.e * H + col0 + j * 16 + l15];
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < NI / 2; ++i) {
             if (wm * 128 + i * 32 >= tc.rows) continue;  // wave-uniform
-            stage_block([&](int j, int r) {
-                return acc[i][j][r] * row_scale[wm * 128 + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3)] * ws[j];
+            stage_block([&](int b, int j, int r) {
+                return acc[2 * i + b][j][r] * row_scale[wm * 128 + i * 32 + b * 16 + g4 * 4 + r] * ws[j];
             });
             for_chunks(i, [&](int trow, int c, u32x4_t v) {
                 const int64_t grow = tc.row0 + trow;
