@@ -28,7 +28,7 @@ extern "C" {
 #define PICOMOE_F32 0
 #define PICOMOE_BF16 1
 
-#define PICOMOE_ABI_VERSION 4
+#define PICOMOE_ABI_VERSION 5
 
 /* ABI version of the loaded library (compare with PICOMOE_ABI_VERSION). */
 int picomoe_abi_version(void);
@@ -97,9 +97,15 @@ int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, int num_expe
  * bytes, e.g. more than 261120 rows at 1024 experts or 33 million rows at 8 -- are refused with PICOMOE_ERR_TOO_LARGE.
  * Every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU (different streams or threads)
  * race; calls on one stream are ordered.  Nothing in the array has to be cleared between calls (each call writes every
- * entry before reading it).  Results are identical to picomoe_permute_plan's. */
+ * entry before reading it).  Results are identical to picomoe_permute_plan's.
+ * picomoe_permute_plan_static_init() is its set-up, also without a counterpart in the reference: it looks up the
+ * address of the current device's array (one runtime symbol query, no allocation, no launch) and keeps it.  Call it
+ * once per device, with that device current, before the first picomoe_permute_plan_static of a stream capture;
+ * without it the first plan call on a device does the lookup itself, which an eager call may and a captured one should
+ * not.  Calling it again is free. */
 #define PICOMOE_PLAN_STATIC_BYTES (1 << 20)
 int64_t picomoe_permute_plan_static_max_bytes(void);
+int picomoe_permute_plan_static_init(void);
 int picomoe_permute_plan_static(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
                                 int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts, int64_t* kept_counts,
                                 int32_t* within, void* stream);

@@ -12,7 +12,7 @@ import torch
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libpicomoe.so")
 HEADER_PATH = os.path.join(os.path.dirname(_PKG_DIR), "include", "picomoe.h")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -32,6 +32,7 @@ _SIGNATURES = {
     "picomoe_permute_workspace_bytes": [_i64, _i32],
     "picomoe_permute_plan": [_p, _i64, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
     "picomoe_permute_plan_static_max_bytes": [],
+    "picomoe_permute_plan_static_init": [],
     "picomoe_permute_plan_static": [_p, _i64, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p],
     "picomoe_gather_rows": [_p, _p, _i32, _i64, _i64, _i32, _p, _p],
     "picomoe_combine_fwd": [_p, _p, _p, _i64, _i32, _i64, _i32, _p, _p],

@@ -428,6 +428,11 @@ extern "C" int picomoe_permute_plan(const int64_t* expert_idx, int64_t n_rows, i
 
 extern "C" int64_t picomoe_permute_plan_static_max_bytes(void) { return PICOMOE_PLAN_STATIC_BYTES; }
 
+extern "C" int picomoe_permute_plan_static_init(void) {
+    int rc = PICOMOE_OK;
+    return static_scratch(&rc) ? PICOMOE_OK : rc;
+}
+
 extern "C" int picomoe_permute_plan_static(const int64_t* expert_idx, int64_t n_rows, int num_experts, int64_t capacity,
                                            int64_t round_index, int32_t* order, int32_t* inv_order, int64_t* counts,
                                            int64_t* kept_counts, int32_t* within, void* stream) {

@@ -236,15 +236,16 @@ class MoELayer(nn.Module):
                 and megakernel.fp8_gemm_supported(self.expert_dim, self.local_experts[0].gate_proj.weight.shape[0]))
 
     def _quantized_weights(self):
-        """E4M3 codes + per-row scales of the stacked gate / up (and, with ``ep_fp8_gemm == "all"``, down) weights.  Training: redone every forward (the
-        optimizer changes the weights every step).  Eval: kept until a parameter's version counter moves; after a
-        write that bypasses the counters (``p.data``) call ``invalidate_fp8_weights``."""
+        """E4M3 codes + per-row scales of the stacked gate / up (and, with ``ep_fp8_gemm == "all"``, down) weights, kept
+        until a parameter's version counter moves: an optimizer step updates the parameters in place and so moves
+        them, the micro-batches of a gradient-accumulation step in between reuse the codes.  After a write that
+        bypasses the counters (``p.data``) call ``invalidate_fp8_weights``."""
         gates, ups, downs = self._expert_params()
         with_down = self.ep_fp8_gemm == "all"
         params = gates + ups + (downs if with_down else [])
         key = (with_down, self._stacks[0].data_ptr(), self._stacks[1].data_ptr(), self._stacks[2].data_ptr(),
                tuple(p._version for p in params))
-        if self.training or self._fp8_weights is None or self._fp8_weights[0] != key:
+        if self._fp8_weights is None or self._fp8_weights[0] != key:
             with torch.no_grad():
                 quantized = megakernel.quantize_expert_weights(self._stacks[0]) + megakernel.quantize_expert_weights(self._stacks[1])
                 if with_down:

@@ -119,9 +119,11 @@ def test_explicit_dgrad_wgrad_api(gpu, dtype):
     g13 = torch.cat([torch.einsum("nh,nih->ni", xf, gf[owner]), torch.einsum("nh,nih->ni", xf, uf[owner])], 1)
     ra = torch.nn.functional.silu(g13[:, :I]) * g13[:, I:]
     rd13 = O.silu_and_mul_bwd(g13, torch.einsum("nh,nhi->ni", dyf, df[owner]))
-    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=5e-2, atol=5e-2)
     for got, want in ((dx, rdx), (a, ra), (d13, rd13), (dg, rdg), (du, rdu), (dd, rdd)):
-        assert torch.allclose(got.cpu().float(), want, **tol)
+        if dtype == torch.float32:
+            assert torch.allclose(got.cpu().float(), want, rtol=1e-4, atol=1e-5)
+        else:  # bf16: every element within 1e-2 of the tensor's scale, the bar of the ragged tests below
+            assert (got.cpu().float() - want).abs().max().item() <= 1e-2 * want.abs().max().item()
 
 
 @pytest.mark.parametrize("H,I,counts", [(256, 512, [130, 128, 126, 0, 1, 64, 63, 0]), (100, 36, [7, 300]), (256, 384, [300, 0, 5, 257]), (512, 128, [1, 1000, 70]),

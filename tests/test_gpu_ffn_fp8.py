@@ -158,6 +158,46 @@ def test_fp8_down_against_bf16_down(gpu):
     assert (y - ref).abs().max().item() <= 5e-2 * ref.abs().max().item()
 
 
+def test_fp8_rows_past_the_segments(gpu):
+    """n_rows > sum(counts) for the two FP8 entry points, as in the capacity modes: the slack rows of the code buffers
+    hold 0x7F (the E4M3 NaN code) with NaN scales, the slack rows of the outputs are pre-filled.  Valid rows must equal
+    the run without slack bit for bit and the slack rows of act, [g|u] and y must come back untouched."""
+    from picotron_amd import _lib
+    from picotron_amd.expert_parallel import megakernel as mk
+
+    lib = _lib.load()
+    E, H, I, counts = 4, 256, 384, [70, 0, 300, 129]
+    n = sum(counts)
+    x, cnt, gw, uw = _mk(E, H, I, counts, seed=21)
+    act_in, _, dw, rw = _mk_down(E, H, I, counts, seed=22)
+    xq, xs = mk._quantize_rows(x.cuda())
+    aq, a_s = mk._quantize_rows(act_in.cuda())
+    gq, gs = mk.quantize_expert_weights(gw.cuda())
+    uq, us = mk.quantize_expert_weights(uw.cuda())
+    dq, ds = mk.quantize_expert_weights(dw.cuda())
+    cntd, rwd, st, P = cnt.cuda(), rw.cuda(), _lib.stream_ptr(), _lib.ptr
+
+    def run(slack):
+        N = n + slack
+        codes = lambda q: torch.cat([q, torch.full((slack, q.shape[1]), 0x7F, dtype=torch.uint8, device="cuda")])
+        scales = lambda s_: torch.cat([s_, torch.full((slack,), float("nan"), device="cuda")])
+        fill = lambda cols: torch.full((N, cols), 7.0, dtype=torch.bfloat16, device="cuda")
+        act, i13, y = fill(I), fill(2 * I), fill(H)
+        _lib.check(lib.picomoe_ffn_gate_up_fp8(P(codes(xq)), P(scales(xs)), P(cntd), E, N, H, I, P(gq), P(uq), P(gs), P(us),
+                                               P(act), P(i13), st), "gate_up_fp8")
+        rwp = torch.cat([rwd, torch.full((slack,), float("nan"), dtype=torch.bfloat16, device="cuda")])
+        _lib.check(lib.picomoe_ffn_down_fp8(P(codes(aq)), P(scales(a_s)), P(cntd), E, N, H, I, P(dq), P(ds), P(rwp), P(y), st),
+                   "down_fp8")
+        torch.cuda.synchronize()
+        return {"act": act, "inter13": i13, "y": y}
+
+    base, padded = run(0), run(37)
+    for name, t in padded.items():
+        assert torch.isfinite(t[:n]).all(), name
+        assert torch.equal(t[:n], base[name]), name
+        assert torch.all(t[n:] == 7.0), name
+
+
 def test_fp8_gate_up_rejects_untiled_shapes(gpu):
     from picotron_amd import _lib
     from picotron_amd.expert_parallel import megakernel as mk
@@ -174,10 +214,19 @@ def test_fp8_gate_up_rejects_untiled_shapes(gpu):
 @pytest.mark.parametrize("mode", [True, "all"])
 def test_layer_with_fp8_gemm(gpu, mode):
     """MoELayer, FP8 dispatch + FP8 gate/up GEMM (``True``) or FP8 gate/up and down GEMMs (``"all"``), forward and
-    backward: outputs within the FP8 tolerance of the oracle's layer with FP8 dispatch (bf16 GEMMs on dequantised
-    rows); same routing; gradients (bf16 backward kernels through the FP8 forward's intermediates) within the same
-    tolerance of the layer without the FP8 GEMM.  With both GEMMs on FP8 their quantisation noises add in quadrature:
-    each is held to relative L2 0.05 on its own (tests above), the chain of the two to 0.05 * sqrt(2)."""
+    backward, against the oracle's layer with FP8 dispatch (bf16 GEMMs on the dequantised rows, unquantised weights,
+    gradients by its autograd): same routing; the output, d x and every parameter gradient within the FP8 tolerance,
+    relative L2 < 0.05 and 5e-2 of the tensor's scale elementwise.  (The backward runs the bf16 kernels on the FP8
+    forward's intermediates, which the down GEMM's mode does not change.)
+
+    One exception, stated rather than hidden: the *output* of ``"all"`` is outside the 5e-2 contract.  E4M3 keeps three
+    mantissa bits, a relative rounding error of about 2.6e-2 rms per quantised operand.  Quantising the gate and the up
+    weights puts 3.8e-2 on the SwiGLU output (measured here with ``True``: the dominant term); quantising that output
+    per row and the down weights per row adds two more terms of 2.4e-2 each, and the three add in quadrature to
+    5.1e-2 -- measured 5.07e-2 relative L2 and 6.1e-2 of the scale in the worst element.  No scale granularity changes
+    that (the noise is the mantissa's), so ``"all"`` stays an opt-in outside the contract; its output and the two
+    gradients that are functions of it (the router's, through d gate-weight = <dy, y>, and d x through the router) are
+    held here to 7.5e-2 only as a guard against gross errors."""
     import types
 
     from picotron_amd.expert_parallel.expert_parallel import MoELayer
@@ -198,9 +247,9 @@ def test_layer_with_fp8_gemm(gpu, mode):
         moe.zero_grad(set_to_none=True)
         xin = x.cuda().requires_grad_(True)
         out = moe(xin)
-        (out.float() * up.cuda().float()).sum().backward()
+        out.backward(up.cuda())
         grads = {n: p.grad.float().cpu() for n, p in moe.named_parameters()}
-        return out.detach().float().cpu(), xin.grad.float().cpu(), grads
+        return out.detach().float().cpu()[0], xin.grad.float().cpu()[0], grads
 
     out8, dx8, g8 = run(mode)
     out16, dx16, g16 = run(False)
@@ -210,24 +259,47 @@ def test_layer_with_fp8_gemm(gpu, mode):
         up_w=torch.stack([e.up_proj.weight.detach().cpu() for e in moe.local_experts]),
         down_w=torch.stack([e.down_proj.weight.detach().cpu() for e in moe.local_experts]),
     )
-    ref, _ = O.moe_forward(x[0], w, k, fp8_dispatch=True)
-    ref = ref.float()
-    assert ((out16[0] - ref).norm() / ref.norm()).item() < 1e-2            # the bf16 path, for scale
-    bound = 0.05 if mode is True else 0.05 * 2 ** 0.5
-    assert ((out8[0] - ref).norm() / ref.norm()).item() < bound
-    assert (out8[0] - ref).abs().max().item() <= bound * ref.abs().max().item()
-    assert ((dx8 - dx16).norm() / dx16.norm()).item() < 0.05
-    for name in g16:
-        if g16[name].norm() > 0:
-            assert ((g8[name] - g16[name]).norm() / g16[name].norm()).item() < 0.05, name
-    # eval mode keeps the quantised weights until a parameter changes
-    moe.eval()
-    moe.ep_fp8_gemm = mode
+    for t in w.tensors():
+        t.requires_grad_(True)
+    xr = x[0].clone().requires_grad_(True)
     with torch.no_grad():
-        a = moe(x.cuda())
-        cached = moe._fp8_weights[1][0].data_ptr()
-        b = moe(x.cuda())
-        assert moe._fp8_weights[1][0].data_ptr() == cached and torch.equal(a, b)
-        moe.local_experts[0].gate_proj.weight.mul_(2.0)
-        c = moe(x.cuda())
-        assert not torch.equal(a, c)
+        logits = moe.gate(x.cuda()[0]).cpu()     # the GPU's logit values: a rounding flip of a near-tie would change the routing
+    own = torch.nn.functional.linear(xr, w.router_w)
+    ref, info = O.moe_forward(xr, w, k, logits=(own.float() + (logits.float() - own.float()).detach()).to(own.dtype), fp8_dispatch=True)
+    ref.backward(up[0])
+    want = {"gate.weight": w.router_w.grad.float()}
+    for e in range(E):
+        for name, t in (("gate_proj", w.gate_w), ("up_proj", w.up_w), ("down_proj", w.down_w)):
+            want[f"local_experts.{e}.{name}.weight"] = t.grad[e].float()
+    ref = ref.detach().float()
+
+    def within(got, ref_t, bound, what):
+        rel = ((got - ref_t).norm() / ref_t.norm()).item()
+        worst = (got - ref_t).abs().max().item() / ref_t.abs().max().item()
+        print(f"[{mode}] {what:36s} rel-L2 {rel:.2e}  max-element {worst:.2e}", flush=True)
+        assert rel < bound and worst <= bound, (what, rel, worst)
+
+    within(out16, ref, 1e-2, "out (bf16 GEMMs, for scale)")
+    loose = 0.05 if mode is True else 0.075
+    within(out8, ref, loose, "out")
+    within(dx8, xr.grad.float(), loose, "d x")
+    assert set(g8) == set(want)
+    for name in sorted(want):
+        if want[name].norm() > 0:
+            within(g8[name], want[name], loose if name == "gate.weight" else 0.05, "d " + name)
+    # the quantised weights are kept until a parameter changes, in training mode too (the micro-batches of a
+    # gradient-accumulation step share them); an in-place update, which is what an optimizer step is, renews them
+    for training in (True, False):
+        moe.train(training)
+        moe.ep_fp8_gemm = mode
+        moe.invalidate_fp8_weights()
+        with torch.no_grad():
+            a = moe(x.cuda())
+            cached = moe._fp8_weights[1][0].data_ptr()
+            b = moe(x.cuda())
+            assert moe._fp8_weights[1][0].data_ptr() == cached and torch.equal(a, b)
+            moe.local_experts[0].gate_proj.weight.mul_(2.0)
+            c = moe(x.cuda())
+            assert moe._fp8_weights[1][0].data_ptr() != cached or not torch.equal(a, c)
+            assert not torch.equal(a, c)
+            moe.local_experts[0].gate_proj.weight.mul_(0.5)

@@ -116,27 +116,49 @@ def test_training_steps_follow_the_oracle_fp32(gpu):
 
 
 def test_bf16_mfma_shapes_forward_backward(gpu):
-    """bf16 with expert shapes the MFMA kernels take (H 256, I 128): logits and gradients within the bf16 tolerance of
-    the oracle run in bf16 on the CPU (relative L2; a token whose router scores nearly tie may pick another expert)."""
+    """bf16 with expert shapes the MFMA kernels take (H 256, I 128): logits and gradients against the oracle.
+
+    Why the bars are wider than the single layer's 1e-2: the oracle run in bf16 on the CPU is itself one bf16
+    evaluation of a 4-layer decoder -- 4 x (attention + MoE) with a rounding after every op, library kernels (attention,
+    norms, dense projections) that round in other places on the GPU than on the CPU, a router whose near-tie tokens
+    may pick another expert once the hidden state differs in its last bit, and a backward pass through all of it -- so
+    two correct bf16 evaluations differ by a few rounding steps per layer.  The test therefore measures both bf16
+    evaluations against the same oracle evaluated in fp32 arithmetic on the same bf16 weights (the value both
+    approximate) and requires the GPU model to be about as close to it as the CPU's bf16 evaluation is (within a factor
+    of 2 plus 5e-3); the direct GPU-vs-CPU-bf16 bars (logits 2e-2, loss 5e-2, gradients 6e-2 relative L2) are kept as
+    a gross-error check."""
     cfg = make_config(hidden_size=256, intermediate_size=128, vocab_size=512, max_position_embeddings=128,
                       router_aux_loss_coef=0.01)
     model = build(cfg, seed=8, dtype=torch.bfloat16, std=0.05).train()
     sd = cpu_state(model, grad=True)
+    sd32 = {k: v.detach().float().requires_grad_(v.requires_grad) for k, v in sd.items()}
     ids, tgt = batch(cfg, 2, 128, seed=9)
     from picotron_amd.expert_parallel.expert_parallel import collect_aux_loss
 
     logits = model(ids.cuda())
     loss = F.cross_entropy(logits.view(-1, logits.size(-1)).float(), tgt.cuda().view(-1))
     (loss + collect_aux_loss(model).float()).backward()
+    rel_l2 = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()
     ref_logits, _ = L.llama_forward({k: v.detach() for k, v in sd.items()}, cfg, ids, training=False)
-    rel = ((logits.detach().float().cpu() - ref_logits.float()).norm() / ref_logits.float().norm()).item()
+    true_logits, _ = L.llama_forward({k: v.detach() for k, v in sd32.items()}, cfg, ids, training=False)
+    got_logits = logits.detach().cpu()
+    rel = rel_l2(got_logits, ref_logits)
     assert rel < 2e-2, rel
+    e_gpu, e_cpu = rel_l2(got_logits, true_logits), rel_l2(ref_logits, true_logits)
+    print(f"logits vs the fp32 evaluation: GPU bf16 {e_gpu:.2e}, CPU bf16 {e_cpu:.2e}", flush=True)
+    assert e_gpu <= 2.0 * e_cpu + 5e-3, (e_gpu, e_cpu)
     ref = L.train_loss(sd, cfg, ids, tgt)
     ref.backward()
+    true = L.train_loss(sd32, cfg, ids, tgt)
+    true.backward()
     assert abs(float(loss.detach()) - float(ref.detach())) < 5e-2 * abs(float(ref.detach()))
     for k, p in model.named_parameters():
         r = sd[k].grad.float()
         if float(r.norm()) == 0.0:
             continue
-        rel = ((p.grad.float().cpu() - r).norm() / r.norm()).item()
+        rel = rel_l2(p.grad.cpu(), r)
         assert rel < 6e-2, (k, rel)
+        t = sd32[k].grad
+        e_gpu, e_cpu = rel_l2(p.grad.cpu(), t), rel_l2(r, t)
+        print(f"d {k:48s} vs fp32: GPU bf16 {e_gpu:.2e}, CPU bf16 {e_cpu:.2e}", flush=True)
+        assert e_gpu <= 2.0 * e_cpu + 5e-3, (k, e_gpu, e_cpu)
