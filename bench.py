@@ -254,6 +254,14 @@ def fp8_gemm_variant(moe, step, w, steps):
         setattr(mk, n, wrap(n, orig[n]))
     rows = w["T"] * w["k"]
     out = {}
+    layer_step = step
+
+    def step():
+        # a training step ends in an optimizer update, which changes every weight: the cached codes are dropped as that
+        # update would drop them, so the weight quantisation is inside every timed step
+        moe.invalidate_fp8_weights()
+        layer_step()
+
     try:
         for mode in (True, "all"):
             moe.ep_fp8_gemm = mode
@@ -298,6 +306,59 @@ def fp8_gemm_variant(moe, step, w, steps):
         for n in names:
             setattr(mk, n, orig[n])
     return out
+
+
+MFMA_NOMINAL_CLOCK_GHZ = 2.4   # the shader clock the datasheet peaks are quoted at
+
+
+def mfma_ceiling(device, launches=8):
+    """What the matrix pipes sustain on this box under its power limit: the library's MFMA-only loop
+    (`picomoe_diag_mfma_loop`: one block of 8 wavefronts per CU, 32 independent accumulator blocks per wavefront, no
+    memory traffic inside the loop) on random operands, and on all-zero operands for scale.  TFLOP/s per MFMA shape,
+    each from `launches` back-to-back launches of about 5 ms between two events on the launch stream."""
+    import torch
+
+    from picotron_amd import _lib
+
+    lib = _lib.load()
+    n_blocks = torch.cuda.get_device_properties(device).multi_processor_count
+    g = torch.Generator(device=device).manual_seed(7)
+    rand16 = torch.randn(8 << 20, generator=g, device=device).bfloat16()
+    # random E4M3 codes, the two NaN codes (0x7F, 0xFF) replaced by 1.0
+    rand8 = torch.randint(0, 256, (16 << 20,), generator=g, device=device, dtype=torch.int16).to(torch.uint8)
+    rand8 = torch.where((rand8 & 0x7F) == 0x7F, torch.full_like(rand8, 0x38), rand8)
+    zeros = torch.zeros(16 << 20, dtype=torch.uint8, device=device)
+    st = _lib.stream_ptr()
+    out = {}
+    for name, shape, data, iters in (("bf16_16x16x32", 0, rand16, 5000), ("bf16_32x32x16", 1, rand16, 5000),
+                                     ("fp8_16x16x128", 2, rand8, 5000), ("bf16_16x16x32_zero_operands", 0, zeros, 5000)):
+        nbytes = data.numel() * data.element_size()
+        flop = lib.picomoe_diag_mfma_loop_flop(shape, iters, n_blocks)
+
+        def launch():
+            _lib.check(lib.picomoe_diag_mfma_loop(_lib.ptr(data), nbytes, shape, iters, n_blocks, None, st), "picomoe_diag_mfma_loop")
+
+        ms = time_events(launch, launches, warm=3)
+        out[name] = flop / ms / 1e9
+    return out, n_blocks
+
+
+def hipblaslt_dense(device, rows, H, I, iters=10):
+    """The vendor comparator: the gate/up and the down GEMM of the layer as ONE dense library GEMM each over all routed
+    rows (one weight matrix instead of one per expert, no SwiGLU, no ragged segments), `torch.nn.functional.linear` =
+    hipBLASLt, on N(0, 1) activations and N(0, 0.02) weights.  TFLOP/s."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(8)
+    x = torch.randn(rows, H, generator=g, device=device).bfloat16()
+    w13 = (0.02 * torch.randn(2 * I, H, generator=g, device=device)).bfloat16()
+    t_gu = time_events(lambda: torch.nn.functional.linear(x, w13), iters, warm=3)
+    del w13, x
+    act = torch.randn(rows, I, generator=g, device=device).bfloat16()
+    w2 = (0.02 * torch.randn(H, I, generator=g, device=device)).bfloat16()
+    t_d = time_events(lambda: torch.nn.functional.linear(act, w2), iters, warm=3)
+    return {"gate_up": 4.0 * rows * H * I / t_gu / 1e9, "down": 2.0 * rows * H * I / t_d / 1e9,
+            "gate_up_ms": t_gu, "down_ms": t_d}
 
 
 def cpu_baseline(w, moe, budget_s=25.0):
@@ -613,6 +674,22 @@ def main():
         }
         log(f"[bench] grouped GEMM: {achieved:.0f} TFLOP/s over {total_ms:.2f} ms/step "
             + " ".join(f"{k}={t:.2f}ms" for k, (t, _) in kt.items()))
+        # the ceiling the power limit leaves on this box, and the vendor library's dense GEMMs of the same sizes
+        ceiling, n_cus = mfma_ceiling(device)
+        dense = hipblaslt_dense(device, w["T"] * w["k"], w["H"], w["I"])
+        best = ceiling["bf16_16x16x32"]
+        result["roofline"].update({
+            "power_capped_mfma_tflops": best,
+            "power_capped_mfma": {"tflops": ceiling, "cus": n_cus,
+                                  "implied_clock_ghz": MFMA_NOMINAL_CLOCK_GHZ * best / MFMA_BF16_PEAK_TFLOPS,
+                                  "what": "picomoe_diag_mfma_loop: MFMA-only loop, 8 wavefronts per CU, random bf16 operands"},
+            "frac_of_power_capped_mfma": achieved / best,
+            "hipblaslt_dense_tflops": {k: dense[k] for k in ("gate_up", "down")},
+            "hipblaslt_dense": {**dense, "what": "torch.nn.functional.linear (hipBLASLt), one dense GEMM over all routed rows "
+                                                 "against one expert's weight matrix: x @ [gate_w; up_w].T and act @ down_w.T"},
+        })
+        log(f"[bench] MFMA-only loop under the power limit: " + ", ".join(f"{k} {v:.0f}" for k, v in ceiling.items())
+            + f" TFLOP/s; hipBLASLt dense gate_up {dense['gate_up']:.0f}, down {dense['down']:.0f} TFLOP/s")
         qg, dg, tq, td = fp8_quant_bandwidth(device)
         result["fp8_quant"] = {"GBps": qg, "frac_hbm": qg / HBM_PEAK_GBPS, "us": tq, "dequant_GBps": dg,
                                "dequant_frac_hbm": dg / HBM_PEAK_GBPS, "dequant_us": td,

@@ -47,6 +47,19 @@ int picomoe_fp8_quant(const void* x, int dtype, int64_t n_rows, int64_t hidden, 
 int picomoe_fp8_dequant(const uint8_t* q, const float* scale, int64_t n_rows, int64_t hidden, void* out, int dtype,
                         void* stream);
 
+/* The FP8 dispatch of one rank in one pass.  Replaces, together, the quantise and the dequantise around the exchange
+ * (EP/ep_communications.py:89-100; with one rank there is no exchange) and the two gathers that expand the tokens to
+ * routed rows and sort them by expert (EP/expert_parallel.py:216-217, :340): every token row is read once and
+ * x_sorted[inv_order[t * top_k + j]] = dequantise(quantise(tokens[t])) for j < top_k, with the arithmetic of
+ * picomoe_fp8_quant and picomoe_fp8_dequant (same codes, same scales, same rounding).  inv_order [n_tokens * top_k] is
+ * the plan's (sorted position of each routed row; negative or >= n_out = not kept: skipped); x_sorted [n_out, hidden]
+ * in dtype.  Optional, both or neither of a pair: q_sorted [n_out, hidden] codes + scale_sorted [n_out] fp32 in the same
+ * order (the operands of picomoe_ffn_gate_up_fp8); q [n_tokens, hidden] + scale [n_tokens] in token order (the wire
+ * format of :63-68).  top_k <= 16. */
+int picomoe_dispatch_fp8(const void* tokens, int dtype, int64_t n_tokens, int64_t hidden, const int32_t* inv_order, int top_k,
+                         int64_t n_out, void* x_sorted, uint8_t* q_sorted, float* scale_sorted, uint8_t* q, float* scale,
+                         void* stream);
+
 /* ---- Router --------------------------------------------------------------------------------------
  * Replaces EP/expert_parallel.py:175-184 (MoELayer._route after the gate Linear): probs =
  * softmax_fp32(logits [n_tokens, num_experts]); picks = top_k of (probs + expert_bias) ordered by
@@ -175,11 +188,36 @@ int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_ex
  * with NULL (or fewer bytes) every tile is computed whole.  Results agree to the rounding of the fp32 partial sums.
  * Calls that overlap in time on different streams need a workspace each. */
 int64_t picomoe_ffn_workspace_bytes(void);
+/* Which kernels the five expert-FFN entry points run for a dtype and layer widths (a query, no launch):
+ * PICOMOE_FFN_BF16_MFMA -- bf16, hidden and inter multiples of 64 and >= 128: 256 x 256 tiles on v_mfma_f32_16x16x32_bf16;
+ * PICOMOE_FFN_F32_MFMA  -- fp32, hidden and inter multiples of 4 and >= 32: 128 x 128 tiles on v_mfma_f32_32x32x2_f32
+ *                          (full fp32 products: the reference runs fp32 inputs on its matrix units too, EP/megakernel.py:162);
+ * PICOMOE_FFN_GENERIC   -- everything else: 64 x 64 tiles of scalar fp32 FMAs, correct for any shape and far slower.
+ * picomoe_ffn_wgrad picks by its own p_dim / q_dim / strides in the same way. */
+#define PICOMOE_FFN_GENERIC 0
+#define PICOMOE_FFN_BF16_MFMA 1
+#define PICOMOE_FFN_F32_MFMA 2
+int picomoe_ffn_kernel_family(int dtype, int64_t hidden, int64_t inter);
 /* Replaces _grouped_wgrad (EP/megakernel.py:209-291): out [E, p_dim, q_dim] with out[e] = lhs_e^T @ rhs_e over the
  * rows of expert e; lhs [n_rows, >=p_dim] with row stride ld_lhs, rhs likewise (so the two halves of d_inter13
  * are addressed in place).  Empty experts get zeros. */
 int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, const int64_t* counts,
                       int num_experts, int64_t n_rows, int64_t p_dim, int64_t q_dim, int dtype, void* out, void* stream);
+
+/* ---- Diagnostics -----------------------------------------------------------------------------------------
+ * No counterpart in the reference and not part of the MoE path: a loop of nothing but MFMAs, to measure what the matrix
+ * pipes sustain under this GPU's power limit -- the ceiling the grouped-GEMM kernels are compared with next to the
+ * datasheet peak.  n_blocks blocks of 8 wavefronts (one block per CU fills the chip with two wavefronts per SIMD), each
+ * wavefront multiplying the same operand fragments into 32 independent accumulator blocks `iters` times.  The fragments
+ * are read once from `operands` (operand_bytes >= 16, 16-byte aligned; indices wrap), so the caller chooses the bit
+ * patterns: random values draw more power than zeros.  `sink` may be NULL.
+ * picomoe_diag_mfma_loop_flop returns the FLOP one such launch performs (-1 for an unknown shape). */
+#define PICOMOE_DIAG_BF16_16X16X32 0 /* v_mfma_f32_16x16x32_bf16 */
+#define PICOMOE_DIAG_BF16_32X32X16 1 /* v_mfma_f32_32x32x16_bf16 */
+#define PICOMOE_DIAG_FP8_16X16X128 2 /* v_mfma_f32_16x16x128_f8f6f4 on E4M3 codes */
+int64_t picomoe_diag_mfma_loop_flop(int shape, int64_t iters, int n_blocks);
+int picomoe_diag_mfma_loop(const void* operands, int64_t operand_bytes, int shape, int64_t iters, int n_blocks, float* sink,
+                           void* stream);
 
 #ifdef __cplusplus
 }

@@ -25,6 +25,7 @@ _SIGNATURES = {
     "picomoe_error_string": [_i32],
     "picomoe_fp8_quant": [_p, _i32, _i64, _i64, _p, _p, _p],
     "picomoe_fp8_dequant": [_p, _p, _i64, _i64, _p, _i32, _p],
+    "picomoe_dispatch_fp8": [_p, _i32, _i64, _i64, _p, _i32, _i64, _p, _p, _p, _p, _p, _p],
     "picomoe_route_partials": [_i64, _i32],
     "picomoe_route_fwd": [_p, _i32, _i64, _i32, _i32, _p, _i32, _p, _p, _p, _p, _p, _p],
     "picomoe_route_bwd": [_p, _p, _p, _i32, _i64, _i32, _i32, _i32, _p, _p, _f32, _p, _p],
@@ -44,11 +45,14 @@ _SIGNATURES = {
     "picomoe_ffn_dgrad_act": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
     "picomoe_ffn_dgrad_x": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _i64, _p],
     "picomoe_ffn_workspace_bytes": [],
+    "picomoe_ffn_kernel_family": [_i32, _i64, _i64],
     "picomoe_ffn_wgrad": [_p, _i64, _p, _i64, _p, _i32, _i64, _i64, _i64, _i32, _p, _p],
+    "picomoe_diag_mfma_loop_flop": [_i32, _i64, _i32],
+    "picomoe_diag_mfma_loop": [_p, _i64, _i32, _i64, _i32, _p, _p],
 }
 _RESTYPES = {"picomoe_error_string": ctypes.c_char_p, "picomoe_permute_workspace_bytes": ctypes.c_int64,
              "picomoe_permute_plan_static_max_bytes": ctypes.c_int64,
-             "picomoe_ffn_workspace_bytes": ctypes.c_int64}
+             "picomoe_ffn_workspace_bytes": ctypes.c_int64, "picomoe_diag_mfma_loop_flop": ctypes.c_int64}
 
 _lib = None
 

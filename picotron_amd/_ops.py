@@ -200,6 +200,45 @@ def expand_permute(src, order, inv_order, div, n_out):
     return _ExpandPermute.apply(src, order, inv_order, div, n_out)
 
 
+class _DispatchFp8(torch.autograd.Function):
+    """x_sorted[inv_order[t*k + j]] = dequantise(quantise(tokens[t])) in one pass over the tokens (FP8 E4M3, one scale per
+    token), optionally with the codes and scales in the same sorted order.  Backward: straight through the quantiser,
+    then the gather-sum of the expand + permute: d_tokens[t] = sum_j d_x_sorted[inv_order[t*k + j]]."""
+
+    @staticmethod
+    def forward(ctx, tokens, inv_order, top_k, n_out, with_codes):
+        _lib.require_cuda(tokens, inv_order)
+        lib = _lib.load()
+        tokens = tokens.contiguous()
+        T, H = tokens.shape
+        # every position is written when nothing is dropped; under a capacity window the unkept tail must not hold garbage
+        x_sorted = _empty((n_out, H), tokens.dtype, tokens.device)
+        q_sorted = _empty((n_out, H), torch.uint8, tokens.device) if with_codes else None
+        scale_sorted = _empty((n_out,), torch.float32, tokens.device) if with_codes else None
+        _lib.check(
+            lib.picomoe_dispatch_fp8(_lib.ptr(tokens), _lib.dtype_code(tokens.dtype), T, H, _lib.ptr(inv_order), int(top_k), n_out,
+                                     _lib.ptr(x_sorted), _lib.ptr(q_sorted), _lib.ptr(scale_sorted), None, None, _lib.stream_ptr()),
+            "picomoe_dispatch_fp8",
+        )
+        ctx.save_for_backward(inv_order)
+        ctx.meta = (T, int(top_k))
+        if with_codes:
+            ctx.mark_non_differentiable(q_sorted, scale_sorted)
+            return x_sorted, q_sorted, scale_sorted
+        return x_sorted, None, None
+
+    @staticmethod
+    def backward(ctx, d_x_sorted, _d_q, _d_scale):
+        (inv_order,) = ctx.saved_tensors
+        n_tokens, top_k = ctx.meta
+        return combine_rows(d_x_sorted, inv_order, None, n_tokens, top_k), None, None, None, None
+
+
+def dispatch_fp8(tokens, inv_order, top_k, n_out, with_codes=False):
+    """(x_sorted, q_sorted or None, scale_sorted or None): the FP8 dispatch of one rank fused with expand + permute."""
+    return _DispatchFp8.apply(tokens, inv_order, top_k, n_out, with_codes)
+
+
 class _UnpermuteCombine(torch.autograd.Function):
     """out[t] = sum_j w[t,j] * y[inv_order[t*k+j]] over kept rows (w None: k = 1 plain un-permute)."""
 

@@ -1,6 +1,6 @@
-// Internal interface between the expert-FFN entry points (ffn_api.hip) and the two kernel families:
-// the generic tiled kernels (ffn_simple.hip: any shape, fp32 or bf16 storage, fp32 FMA arithmetic)
-// and the bf16 MFMA kernels (ffn_mfma.hip: aligned shapes).
+// Internal interface between the expert-FFN entry points (ffn_api.hip) and the kernel families:
+// the generic tiled kernels (ffn_simple.hip: any shape, fp32 or bf16 storage, fp32 FMA arithmetic),
+// the bf16 MFMA kernels (ffn_mfma.hip: aligned shapes) and the fp32 MFMA kernels (ffn_f32_mfma.hip).
 #pragma once
 #include "common.h"
 
@@ -42,6 +42,19 @@ int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_
 int64_t ffn_mfma_workspace_bytes();
 int ffn_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, int64_t P, int64_t Q,
                    void* out, hipStream_t st);
+
+// fp32 MFMA family (ffn_f32_mfma.hip: v_mfma_f32_32x32x2_f32, hidden and inter multiples of 4); a call whose tensors are
+// not 16-byte aligned falls through to the generic kernel of the same name.
+bool ffn_f32_mfma_supported(const FfnShape& s);
+bool ffn_f32_mfma_wgrad_supported(int dtype, int64_t P, int64_t Q, int64_t ld_lhs, int64_t ld_rhs, const void* lhs, const void* rhs);
+int ffn_f32_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
+                         hipStream_t st);
+int ffn_f32_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, hipStream_t st);
+int ffn_f32_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, const void* inter13, void* d_inter13,
+                           void* act_out, hipStream_t st);
+int ffn_f32_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx, hipStream_t st);
+int ffn_f32_mfma_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const void* rhs, int64_t ld_rhs, int64_t P, int64_t Q,
+                       void* out, hipStream_t st);
 
 // FP8 (E4M3) MFMA gate/up and down: codes + one fp32 scale per activation row and per weight row (ffn_fp8.hip)
 bool ffn_fp8_supported(const FfnShape& s);

@@ -1,5 +1,5 @@
 // extern "C" entry points of the expert FFN (grouped SwiGLU GEMMs, forward + dgrad + wgrad).
-// Picks the bf16 MFMA kernels when the shape is one they tile, the generic kernels otherwise.
+// Picks the bf16 or fp32 MFMA kernels when the shape is one they tile, the generic kernels otherwise.
 #include "ffn.h"
 
 namespace {
@@ -19,6 +19,7 @@ extern "C" int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(x && gate_w && up_w && act);
     if (ffn_mfma_supported(s)) return ffn_mfma_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
+    if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
     return ffn_simple_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
 }
 
@@ -47,6 +48,14 @@ extern "C" int picomoe_ffn_down_fp8(const void* actq, const float* act_scale, co
 
 extern "C" int64_t picomoe_ffn_workspace_bytes(void) { return ffn_mfma_workspace_bytes(); }
 
+extern "C" int picomoe_ffn_kernel_family(int dtype, int64_t hidden, int64_t inter) {
+    FfnShape s{};
+    s.dtype = dtype; s.H = hidden; s.I = inter;
+    if (ffn_mfma_supported(s)) return PICOMOE_FFN_BF16_MFMA;
+    if (ffn_f32_mfma_supported(s)) return PICOMOE_FFN_F32_MFMA;
+    return PICOMOE_FFN_GENERIC;
+}
+
 extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                                 int64_t inter, const void* down_w, const void* row_weight, int dtype, void* y, void* workspace,
                                 int64_t workspace_bytes, void* stream) {
@@ -55,6 +64,7 @@ extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(act && down_w && y);
     if (ffn_mfma_supported(s)) return ffn_mfma_down(s, act, down_w, row_weight, y, workspace, workspace_bytes, (hipStream_t)stream);
+    if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
     return ffn_simple_down(s, act, down_w, row_weight, y, (hipStream_t)stream);
 }
 
@@ -66,6 +76,7 @@ extern "C" int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int 
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(dy && down_w && inter13 && d_inter13);
     if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
+    if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
     return ffn_simple_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
 }
 
@@ -77,6 +88,7 @@ extern "C" int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts,
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(d_inter13 && gate_w && up_w && dx);
     if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_x(s, d_inter13, gate_w, up_w, dx, workspace, workspace_bytes, (hipStream_t)stream);
+    if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
     return ffn_simple_dgrad_x(s, d_inter13, gate_w, up_w, dx, (hipStream_t)stream);
 }
 
@@ -89,5 +101,7 @@ extern "C" int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rh
     // n_rows == 0 still has to zero-fill the output: every expert is empty
     if (ffn_mfma_wgrad_supported(dtype, p_dim, q_dim, ld_lhs, ld_rhs, lhs, rhs))
         return ffn_mfma_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
+    if (ffn_f32_mfma_wgrad_supported(dtype, p_dim, q_dim, ld_lhs, ld_rhs, lhs, rhs))
+        return ffn_f32_mfma_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
     return ffn_simple_wgrad(s, lhs, ld_lhs, rhs, ld_rhs, p_dim, q_dim, out, (hipStream_t)stream);
 }

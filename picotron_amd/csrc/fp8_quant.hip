@@ -77,9 +77,9 @@ __device__ __forceinline__ void load_row(const u32x4_t* xr, int lane, int chunks
     }
 }
 
-// amax -> scale -> codes of the row in v; lane 0 writes the scale
-template <int CHUNKS, bool FULL>
-__device__ __forceinline__ void quant_row(const u32x4_t (&v)[CHUNKS], int lane, int chunks_per_row, u32x2_t* qr, float* scale_out) {
+// amax -> scale of the bf16 row a wavefront holds in v
+template <int CHUNKS>
+__device__ __forceinline__ RowScale row_scale_bf16(const u32x4_t (&v)[CHUNKS]) {
     typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
     u16x2 m2 = {0, 0};
 #pragma unroll
@@ -100,6 +100,13 @@ __device__ __forceinline__ void quant_row(const u32x4_t (&v)[CHUNKS], int lane, 
     rs.s = bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(amax_bits) / kE4M3Max));
     rs.r = 1.0f / rs.s;
     rs.finite = amax_bits < 0x7F80u;
+    return rs;
+}
+
+// amax -> scale -> codes of the row in v; lane 0 writes the scale
+template <int CHUNKS, bool FULL>
+__device__ __forceinline__ void quant_row(const u32x4_t (&v)[CHUNKS], int lane, int chunks_per_row, u32x2_t* qr, float* scale_out) {
+    const RowScale rs = row_scale_bf16<CHUNKS>(v);
     if (lane == 0) *scale_out = rs.s;
 
 #pragma unroll
@@ -284,7 +291,167 @@ __global__ __launch_bounds__(256) void dequant_generic(const uint8_t* __restrict
     }
 }
 
+// eight E4M3 codes -> eight bf16: float(code) * s is exact in fp32, one rounding to bf16
+__device__ __forceinline__ u32x4_t dequant_chunk_bf16(const u32x2_t& c, float s) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2;
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, false);
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, true);
+    const f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, false);
+    const f32x2 e = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, true);
+    u32x4_t o;
+    o.x = pack_bf16x2(a.x * s, a.y * s);
+    o.y = pack_bf16x2(b.x * s, b.y * s);
+    o.z = pack_bf16x2(d.x * s, d.y * s);
+    o.w = pack_bf16x2(e.x * s, e.y * s);
+    return o;
+}
+
+// ---- one-pass dispatch -----------------------------------------------------------------------
+// One wavefront per token: the row is read once, quantised, dequantised, and the dequantised row (and, when asked for,
+// the codes and the scale) written straight to the sorted positions of the token's top_k routed rows.  HBM sees
+// hidden * 2 bytes read and top_k * hidden * (2 [+ 1]) bytes written per token: what a quantise pass, a dequantise pass
+// and the expand + permute gather(s) move one after the other, without the two intermediate copies.
+constexpr int kDispatchMaxTopK = 16;
+
+template <int CHUNKS, bool FULL>
+__global__ __launch_bounds__(256) void dispatch_bf16_wave_per_token(const u32x4_t* __restrict__ tokens, int64_t n_tokens,
+                                                                    int chunks_per_row, const int32_t* __restrict__ inv_order,
+                                                                    int top_k, int64_t n_out, u32x4_t* __restrict__ x_sorted,
+                                                                    u32x2_t* __restrict__ q_sorted, float* __restrict__ scale_sorted,
+                                                                    u32x2_t* __restrict__ q, float* __restrict__ scale) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tokens) return;  // uniform per wave
+    u32x4_t v[CHUNKS];
+    load_row<CHUNKS, FULL>(tokens + t * chunks_per_row, lane, chunks_per_row, v);
+    // the sorted positions of this token's routed rows: wave-uniform, kept in scalar registers
+    int pos[kDispatchMaxTopK];
+#pragma unroll
+    for (int j = 0; j < kDispatchMaxTopK; ++j) {
+        int p = j < top_k ? inv_order[t * top_k + j] : -1;
+        if (p >= n_out) p = -1;
+        pos[j] = __builtin_amdgcn_readfirstlane(p);
+    }
+    const RowScale rs = row_scale_bf16<CHUNKS>(v);
+    if (lane == 0) {
+        if (scale) scale[t] = rs.s;
+        if (scale_sorted) {
+#pragma unroll
+            for (int j = 0; j < kDispatchMaxTopK; ++j)
+                if (pos[j] >= 0) scale_sorted[pos[j]] = rs.s;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int idx = c * 64 + lane;
+        if (!FULL && idx >= chunks_per_row) continue;
+        const u32x2_t codes = quant_chunk(v[c], rs);
+        const u32x4_t deq = dequant_chunk_bf16(codes, rs.s);
+        if (q) __builtin_nontemporal_store(codes, q + t * chunks_per_row + idx);
+#pragma unroll
+        for (int j = 0; j < kDispatchMaxTopK; ++j) {
+            if (pos[j] < 0) continue;  // wave-uniform
+            __builtin_nontemporal_store(deq, x_sorted + (int64_t)pos[j] * chunks_per_row + idx);
+            if (q_sorted) __builtin_nontemporal_store(codes, q_sorted + (int64_t)pos[j] * chunks_per_row + idx);
+        }
+    }
+}
+
+// Any dtype / width: one block per token, the arithmetic of quant_generic and dequant_generic.
+template <typename T>
+__global__ __launch_bounds__(256) void dispatch_generic(const T* __restrict__ tokens, int64_t hidden,
+                                                        const int32_t* __restrict__ inv_order, int top_k, int64_t n_out,
+                                                        T* __restrict__ x_sorted, uint8_t* __restrict__ q_sorted,
+                                                        float* __restrict__ scale_sorted, uint8_t* __restrict__ q,
+                                                        float* __restrict__ scale) {
+    __shared__ uint32_t part[4];
+    const int64_t t = blockIdx.x;
+    const T* xr = tokens + t * hidden;
+    uint32_t m = 0;
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        uint32_t b = __float_as_uint(load_as_f32<T>(xr + c)) & 0x7FFFFFFFu;
+        m = b > m ? b : m;
+    }
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = part[0];
+    for (int i = 1; i < 4; ++i) m = part[i] > m ? part[i] : m;
+    const bool has_nan = m > 0x7F800000u;
+    float amax = __uint_as_float(m);
+    float s;
+    if (sizeof(T) == 2) {
+        const float floor_v = bf16_bits_to_f32(kAmaxFloorBf16);
+        if (!has_nan && amax < floor_v) amax = floor_v;
+        s = bf16_bits_to_f32(f32_to_bf16_bits(amax / kE4M3Max));
+    } else {
+        if (!has_nan && amax < 1e-4f) amax = 1e-4f;
+        s = amax / kE4M3Max;
+    }
+    if (threadIdx.x == 0 && scale) scale[t] = s;
+    for (int j = threadIdx.x; j < top_k; j += 256) {
+        const int p = inv_order[t * top_k + j];
+        if (p >= 0 && p < n_out && scale_sorted) scale_sorted[p] = s;
+    }
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        float v = load_as_f32<T>(xr + c) / s;
+        v = (v != v) ? v : clamp448(v);
+        const uint32_t code = cvt2<false>(v, v, 0u) & 0xFFu;
+        const float d = __builtin_amdgcn_cvt_f32_fp8((int)code, 0) * s;
+        if (q) q[t * hidden + c] = (uint8_t)code;
+        for (int j = 0; j < top_k; ++j) {
+            const int p = inv_order[t * top_k + j];
+            if (p < 0 || p >= n_out) continue;
+            if (sizeof(T) == 2)
+                ((uint16_t*)x_sorted)[(int64_t)p * hidden + c] = (uint16_t)f32_to_bf16_bits(d);
+            else
+                ((float*)x_sorted)[(int64_t)p * hidden + c] = d;
+            if (q_sorted) q_sorted[(int64_t)p * hidden + c] = (uint8_t)code;
+        }
+    }
+}
+
 }  // namespace
+
+extern "C" int picomoe_dispatch_fp8(const void* tokens, int dtype, int64_t n_tokens, int64_t hidden, const int32_t* inv_order,
+                                    int top_k, int64_t n_out, void* x_sorted, uint8_t* q_sorted, float* scale_sorted,
+                                    uint8_t* q, float* scale, void* stream) {
+    PICOMOE_CHECK_ARG(n_tokens >= 0 && n_tokens < (1ll << 31) && hidden > 0 && n_out >= 0 && n_out < (1ll << 31));
+    PICOMOE_CHECK_ARG((dtype == PICOMOE_F32 || dtype == PICOMOE_BF16) && top_k >= 1 && top_k <= kDispatchMaxTopK);
+    PICOMOE_CHECK_ARG((q_sorted == nullptr) == (scale_sorted == nullptr) && (q == nullptr) == (scale == nullptr));
+    if (n_tokens == 0) return PICOMOE_OK;
+    PICOMOE_CHECK_ARG(tokens && inv_order && (x_sorted || n_out == 0));
+    hipStream_t st = (hipStream_t)stream;
+    const bool aligned = dtype == PICOMOE_BF16 && hidden % 8 == 0 && hidden <= 8192 && (uintptr_t)tokens % 16 == 0 &&
+                         (uintptr_t)x_sorted % 16 == 0 && (uintptr_t)q_sorted % 8 == 0 && (uintptr_t)q % 8 == 0;
+    if (aligned) {
+        const int cpr = (int)(hidden / 8);
+        const int chunks = (cpr + 63) / 64;
+        const dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
+#define PICOMOE_LAUNCH_D(C)                                                                                             \
+    if (cpr == C * 64)                                                                                                  \
+        hipLaunchKernelGGL((dispatch_bf16_wave_per_token<C, true>), grid, block, 0, st, (const u32x4_t*)tokens, n_tokens, \
+                           cpr, inv_order, top_k, n_out, (u32x4_t*)x_sorted, (u32x2_t*)q_sorted, scale_sorted,          \
+                           (u32x2_t*)q, scale);                                                                         \
+    else                                                                                                                \
+        hipLaunchKernelGGL((dispatch_bf16_wave_per_token<C, false>), grid, block, 0, st, (const u32x4_t*)tokens,        \
+                           n_tokens, cpr, inv_order, top_k, n_out, (u32x4_t*)x_sorted, (u32x2_t*)q_sorted,              \
+                           scale_sorted, (u32x2_t*)q, scale)
+        if (chunks <= 1) PICOMOE_LAUNCH_D(1);
+        else if (chunks <= 2) PICOMOE_LAUNCH_D(2);
+        else if (chunks <= 4) PICOMOE_LAUNCH_D(4);
+        else if (chunks <= 8) PICOMOE_LAUNCH_D(8);
+        else PICOMOE_LAUNCH_D(16);
+#undef PICOMOE_LAUNCH_D
+    } else if (dtype == PICOMOE_BF16) {
+        hipLaunchKernelGGL(dispatch_generic<uint16_t>, dim3((unsigned)n_tokens), dim3(256), 0, st, (const uint16_t*)tokens,
+                           hidden, inv_order, top_k, n_out, (uint16_t*)x_sorted, q_sorted, scale_sorted, q, scale);
+    } else {
+        hipLaunchKernelGGL(dispatch_generic<float>, dim3((unsigned)n_tokens), dim3(256), 0, st, (const float*)tokens, hidden,
+                           inv_order, top_k, n_out, (float*)x_sorted, q_sorted, scale_sorted, q, scale);
+    }
+    return picomoe_launch_status();
+}
 
 extern "C" int picomoe_fp8_quant(const void* x, int dtype, int64_t n_rows, int64_t hidden, uint8_t* q, float* scale,
                                  void* stream) {

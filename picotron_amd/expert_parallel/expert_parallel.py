@@ -20,7 +20,6 @@ import torch.nn as nn
 from picotron_amd import _lib, _ops
 from picotron_amd.expert_parallel import megakernel
 from picotron_amd.expert_parallel.capacity_moe import _capped_rounds, compute_capacity
-from picotron_amd.expert_parallel.ep_communications import fp8_round_trip
 from picotron_amd.model import MLP
 
 
@@ -204,16 +203,14 @@ class MoELayer(nn.Module):
         plan = _ops.permute_plan(topk_idx.reshape(-1), self.num_local_experts)
         codes = None
         if self.ep_fp8_dispatch:
-            # one quantise -> dequantise per token equals one per routed row (a row op on identical rows)
-            if self._use_fp8_gemm(latent):
-                latent, q, scale = fp8_round_trip(latent, with_codes=True)
-                # the codes travel like the rows: gathered into expert order (two codes per 16-bit element)
-                q16 = q.view(torch.uint8).view(torch.int16).view(torch.bfloat16)
-                src = torch.div(plan.order, self.top_k, rounding_mode="floor")
-                codes = (_ops.gather_rows(q16, plan.order, self.top_k, n_rows).view(torch.uint8), scale[src])
-            else:
-                latent = fp8_round_trip(latent)
-        x_sorted = _ops.expand_permute(latent, plan.order, plan.inv_order, self.top_k, n_rows)
+            # One pass over the tokens: quantise -> dequantise (one per token equals one per routed row, a row op on
+            # identical rows) written straight to the rows' sorted positions, with the codes beside them for the FP8 GEMM
+            x_sorted, q_sorted, scale_sorted = _ops.dispatch_fp8(latent, plan.inv_order, self.top_k, n_rows,
+                                                                 with_codes=self._use_fp8_gemm(latent))
+            if q_sorted is not None:
+                codes = (q_sorted, scale_sorted)
+        else:
+            x_sorted = _ops.expand_permute(latent, plan.order, plan.inv_order, self.top_k, n_rows)
         y_sorted = self._grouped_experts(x_sorted, plan.counts, codes)
         y = _ops.unpermute_combine(y_sorted, topk_weights, plan.inv_order, plan.order, num_tokens, self.top_k)
         return self._finalize(y, shared)

@@ -13,6 +13,7 @@ autograd path keeps ``[g|u]`` from the forward instead of recomputing it.
 """
 
 import collections
+import warnings
 
 import torch
 import torch.nn.functional as F
@@ -34,12 +35,29 @@ def _counts64(counts, device):
     return counts.to(device=device, dtype=torch.int64).contiguous()
 
 
+_FAMILY_NAMES = {0: "generic", 1: "bf16_mfma", 2: "f32_mfma"}
+_warned_generic = set()
+
+
+def kernel_family(dtype, hidden, inter):
+    """Which kernels the expert FFN runs for this dtype and these widths: "bf16_mfma" (bf16, multiples of 64, >= 128),
+    "f32_mfma" (fp32, multiples of 4, >= 32) or "generic" (scalar-FMA tiles: any shape, far slower)."""
+    return _FAMILY_NAMES[_lib.load().picomoe_ffn_kernel_family(_lib.dtype_code(dtype), int(hidden), int(inter))]
+
+
 def _check_weights(x, gate_w, up_w, down_w):
     E, I, H = gate_w.shape
     if up_w.shape != (E, I, H) or down_w.shape != (E, H, I) or x.shape[1] != H:
         raise _lib.PicomoeError(f"fused_moe: shapes x{tuple(x.shape)} gate{tuple(gate_w.shape)} up{tuple(up_w.shape)} down{tuple(down_w.shape)}")
     if not (x.dtype == gate_w.dtype == up_w.dtype == down_w.dtype):
         raise _lib.PicomoeError("fused_moe: x and the weights must share one dtype")
+    key = (x.dtype, H, I)
+    if key not in _warned_generic and kernel_family(*key) == "generic":
+        _warned_generic.add(key)   # once per shape: the results are the same, only the speed is not
+        warnings.warn(
+            f"picotron_amd: expert FFN with hidden {H}, FFN {I}, {x.dtype} runs the generic scalar-FMA kernels, not the "
+            "matrix pipes (bf16 needs both widths to be multiples of 64 and >= 128, fp32 multiples of 4 and >= 32)",
+            RuntimeWarning, stacklevel=3)
     return E, I, H
 
 

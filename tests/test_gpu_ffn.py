@@ -193,13 +193,15 @@ def test_split_last_round_matches_whole_tiles(gpu, counts, H):
         assert torch.equal(fn(ws).float().cpu(), split)               # fixed summation order: run to run identical
 
 
-@pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (320, 192, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32)])
+@pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (320, 192, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32),
+                                       (18, 10, torch.float32)])
 def test_rows_past_the_segments_are_never_read_into_a_result(gpu, H, I, dtype):
     """n_rows > sum(counts), as in the capacity modes where the buffers are sized for every routed row and only the kept
     rows are laid out: the slack rows of every input hold NaN, the slack rows of every output are pre-filled.  Results
     for the valid rows and all three weight gradients must equal the run without slack bit for bit, and the slack rows
-    of the outputs must come back untouched.  Covers the MFMA kernels (hidden 256; hidden 320 / FFN 192 with a partly
-    filled last tile column) and the generic ones."""
+    of the outputs must come back untouched.  Covers the bf16 MFMA kernels (hidden 256; hidden 320 / FFN 192 with a partly
+    filled last tile column), the fp32 MFMA kernels (hidden 96 / FFN 40 in fp32) and the generic ones (the same widths in
+    bf16; hidden 18 / FFN 10 in fp32)."""
     from picotron_amd import _lib
 
     lib = _lib.load()
@@ -306,3 +308,73 @@ def test_workspace_cache_is_bounded(gpu):
     assert len(mk._workspaces) == mk._MAX_WORKSPACES
     mk.release_workspaces()
     assert len(mk._workspaces) == 0
+
+
+@pytest.mark.parametrize("H,I,counts", [
+    (256, 512, [5, 0, 130, 17, 300, 1, 127, 128]),   # the tiny configuration's widths; tails, an exact tile, an empty expert
+    (132, 68, [7, 300]),                              # widths that are multiples of 4 only: a K tail in every GEMM
+    (64, 36, [129, 64, 1]),                           # fewer output columns than a tile is wide
+    (2048, 128, [33, 0, 200]),                        # a long contraction
+])
+def test_fp32_mfma_against_oracle(gpu, H, I, counts):
+    """fp32 shapes the matrix-pipe kernels take (v_mfma_f32_32x32x2_f32, full fp32 products): forward and all four
+    gradients within 1e-5 of each tensor's scale of the oracle's fp32 arithmetic, the explicit dgrad / wgrad entry points
+    and their intermediates, and the row-weight epilogue with its gradient."""
+    from picotron_amd.expert_parallel import megakernel
+
+    assert megakernel.kernel_family(torch.float32, H, I) == "f32_mfma"
+    E = len(counts)
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.float32, H + I, scale=0.05)
+    dy = torch.randn(x.shape, generator=g)
+    rw = torch.rand(x.shape[0], generator=g)
+
+    def close(got, want, what):
+        err, scale = (got.cpu() - want).abs().max().item(), want.abs().max().item()
+        assert err <= 1e-5 * scale + 1e-9, f"{what}: max error {err:.3e} against a scale of {scale:.3e}"
+
+    for with_rw in (False, True):
+        leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw)] + ([rw.cuda().requires_grad_(True)] if with_rw else [])
+        y = megakernel.fused_moe(leaves[0], cnt.cuda(), leaves[1], leaves[2], leaves[3], row_weight=leaves[4] if with_rw else None)
+        cl = [t.double().requires_grad_(True) for t in (x, gw, uw, dw)] + ([rw.double().requires_grad_(True)] if with_rw else [])
+        yr = O.expert_ffn(cl[0], cnt, cl[1], cl[2], cl[3], cl[4] if with_rw else None)
+        close(y.detach(), yr.detach().float(), "y")
+        y.backward(dy.cuda())
+        yr.backward(dy.double())
+        for a, b, name in zip(leaves, cl, ("dx", "dgate", "dup", "ddown", "drow_weight")):
+            close(a.grad, b.grad.float(), name)
+        for e, c in enumerate(counts):
+            if c == 0:
+                assert torch.all(leaves[1].grad[e] == 0) and torch.all(leaves[3].grad[e] == 0)
+    # the explicit entry points and what they hand on
+    dx, a, d13 = megakernel.fused_moe_dgrad(x.cuda(), cnt.cuda(), gw.cuda(), uw.cuda(), dw.cuda(), dy.cuda())
+    dg, du, dd = megakernel.fused_moe_wgrad(x.cuda(), cnt.cuda(), a, d13, dy.cuda())
+    owner = torch.repeat_interleave(torch.arange(E), cnt)
+    xd, gd, ud, dd_, dyd = (t.double() for t in (x, gw, uw, dw, dy))
+    g13 = torch.cat([torch.einsum("nh,nih->ni", xd, gd[owner]), torch.einsum("nh,nih->ni", xd, ud[owner])], 1)
+    close(a, (torch.nn.functional.silu(g13[:, :I]) * g13[:, I:]).float(), "a")
+    close(d13, O.silu_and_mul_bwd(g13, torch.einsum("nh,nhi->ni", dyd, dd_[owner])).float(), "d_inter13")
+    rdx, rdg, rdu, rdd = O.expert_ffn_backward(xd, cnt, gd, ud, dd_, dyd)
+    for got, want, name in ((dx, rdx, "dx"), (dg, rdg, "dgate"), (du, rdu, "dup"), (dd, rdd, "ddown")):
+        close(got, want.float(), "explicit " + name)
+
+
+def test_kernel_family_and_the_generic_warning(gpu):
+    """Which kernels a shape runs is a query of the library; a shape that lands on the scalar-FMA kernels warns, once."""
+    import warnings
+
+    from picotron_amd.expert_parallel import megakernel
+
+    fam = megakernel.kernel_family
+    assert fam(torch.bfloat16, 4096, 14336) == "bf16_mfma" and fam(torch.bfloat16, 320, 192) == "bf16_mfma"
+    assert fam(torch.bfloat16, 96, 40) == "generic" and fam(torch.bfloat16, 100, 128) == "generic"
+    assert fam(torch.float32, 256, 512) == "f32_mfma" and fam(torch.float32, 36, 68) == "f32_mfma"
+    assert fam(torch.float32, 16, 32) == "generic" and fam(torch.float32, 130, 64) == "generic"
+    x, counts, gw, uw, dw, _ = _mk(2, 24, 40, [3, 9], torch.bfloat16, 7)
+    megakernel._warned_generic.discard((torch.bfloat16, 24, 40))
+    with pytest.warns(RuntimeWarning, match="generic scalar-FMA"):
+        megakernel.fused_moe_forward(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda())
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        megakernel.fused_moe_forward(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda())   # the second call is silent
+        x2, c2, g2, u2, d2, _ = _mk(2, 256, 128, [3, 9], torch.bfloat16, 8)
+        megakernel.fused_moe_forward(x2.cuda(), c2.cuda(), g2.cuda(), u2.cuda(), d2.cuda())      # an MFMA shape never warns

@@ -152,3 +152,112 @@ def test_round_trip_autograd_is_straight_through(gpu):
     g = torch.randn_like(y)
     y.backward(g)
     assert torch.equal(x.grad, g)
+
+
+def _dispatch(x_cpu, inv, k, n_out, gpu, codes=True, wire=True, prefill=None):
+    """picomoe_dispatch_fp8 through the C ABI with caller-owned, pre-filled outputs."""
+    from picotron_amd import _lib
+
+    lib = _lib.load()
+    T, H = x_cpu.shape
+    fill = 7.0 if prefill is None else prefill
+    xs = torch.full((n_out, H), fill, dtype=x_cpu.dtype, device=gpu)
+    qs = torch.full((n_out, H), 0x11, dtype=torch.uint8, device=gpu) if codes else None
+    ss = torch.full((n_out,), fill, dtype=torch.float32, device=gpu) if codes else None
+    q = torch.full((T, H), 0x11, dtype=torch.uint8, device=gpu) if wire else None
+    s = torch.full((T,), fill, dtype=torch.float32, device=gpu) if wire else None
+    P = _lib.ptr
+    xd, invd = x_cpu.to(gpu), inv.to(gpu)     # named: the buffers must outlive the launch
+    _lib.check(lib.picomoe_dispatch_fp8(P(xd), _lib.dtype_code(x_cpu.dtype), T, H, P(invd), k, n_out, P(xs), P(qs),
+                                        P(ss), P(q), P(s), _lib.stream_ptr()), "picomoe_dispatch_fp8")
+    torch.cuda.synchronize()
+    del xd, invd
+    return tuple(t.cpu() if t is not None else None for t in (xs, qs, ss, q, s))
+
+
+@pytest.mark.parametrize("T,H,E,k,dtype", [
+    (512, 4096, 8, 2, torch.bfloat16),     # the Mixtral row width: a wave per token, every chunk round full
+    (300, 2048, 64, 6, torch.bfloat16),    # fine-grained: top-6
+    (129, 1000, 4, 1, torch.bfloat16),     # a partly filled last chunk round, top-1
+    (67, 8192, 8, 16, torch.bfloat16),     # the widest wave-per-token row, the largest top-k
+    (40, 100, 4, 2, torch.bfloat16),       # rows that are not whole 16-byte chunks: the generic kernel
+    (33, 8200, 4, 2, torch.bfloat16),      # rows longer than a wavefront holds: the generic kernel
+    (65, 256, 8, 2, torch.float32),        # fp32 rows
+])
+def test_dispatch_fp8_is_quant_dequant_permute_in_one_pass(gpu, T, H, E, k, dtype):
+    """picomoe_dispatch_fp8 against the oracle's quantise -> dequantise composed with its stable sort by expert:
+    x_sorted == dequant(quant(tokens))[order // k], the sorted codes and scales likewise, the token-order codes and
+    scales equal the quantiser's -- all bit for bit; edge rows (zeros, below the amax floor, huge, infinite) included."""
+    x = _c2_input(T, H, seed=T + H).to(dtype)
+    x[0] = 0
+    x[1] = 1e-6
+    x[2, 3] = 3e38 if dtype == torch.float32 else 3e38
+    x[3, 5] = float("inf")
+    g = torch.Generator().manual_seed(k)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] if k <= E else torch.randint(0, E, (k,), generator=g) for _ in range(T)])
+    order, inv, counts = O.permute_plan_fast(idx.reshape(-1), E)
+    q_ref, s_ref = O.quant_fp8(x)
+    d_ref = O.dequant_fp8(q_ref, s_ref, dtype)
+
+    def bits(t):
+        # bit patterns, with every NaN mapped to one pattern: the row with an infinite entry dequantises to NaN
+        # (0 * inf), and which NaN a platform produces is not part of the contract
+        b = t.view(torch.int16 if t.dtype == torch.bfloat16 else torch.int32)
+        return torch.where(torch.isnan(t), torch.full_like(b, -1), b)
+
+    xs, qs, ss, q, s = _dispatch(x, inv.int(), k, T * k, gpu)
+    src = order // k
+    assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
+    assert torch.isnan(d_ref[3]).all() and not torch.isnan(d_ref[:3]).any() and not torch.isnan(d_ref[4:]).any()
+    assert torch.equal(bits(xs), bits(d_ref[src]))
+    assert torch.equal(qs, q_ref[src]) and torch.equal(ss.view(torch.int32), s_ref[src].view(torch.int32))
+    # without the optional outputs: the same rows
+    xs2, _, _, _, _ = _dispatch(x, inv.int(), k, T * k, gpu, codes=False, wire=False)
+    assert torch.equal(bits(xs2), bits(xs))
+    # and it equals the three-pass form it replaces, kernel for kernel
+    from picotron_amd import _ops
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    three = _ops.gather_rows(C.fp8_round_trip(x.to(gpu)), order.int().to(gpu), k, T * k)
+    assert torch.equal(bits(three.cpu()), bits(xs))
+
+
+def test_dispatch_fp8_skips_rows_that_are_not_kept(gpu):
+    """Negative positions (rows a capacity window dropped) and positions past n_out are skipped; what no kept row maps to
+    is left as the caller filled it."""
+    T, H, k = 50, 512, 2
+    x = _c2_input(T, H, seed=3).bfloat16()
+    g = torch.Generator().manual_seed(1)
+    n_out = 70
+    perm = torch.randperm(T * k, generator=g)
+    inv = torch.full((T * k,), -1, dtype=torch.int32)
+    inv[perm[:n_out]] = torch.arange(n_out, dtype=torch.int32)       # 70 kept rows, 30 dropped
+    inv[perm[n_out]] = n_out + 5                                      # a position past the buffer: skipped too
+    xs, qs, ss, _, _ = _dispatch(x, inv, k, n_out + 4, gpu)
+    q_ref, s_ref = O.quant_fp8(x)
+    d_ref = O.dequant_fp8(q_ref, s_ref, torch.bfloat16)
+    src = perm[:n_out] // k
+    assert torch.equal(xs[:n_out].view(torch.int16), d_ref[src].view(torch.int16))
+    assert torch.equal(qs[:n_out], q_ref[src]) and torch.equal(ss[:n_out], s_ref[src])
+    assert torch.all(xs[n_out:] == 7.0) and torch.all(qs[n_out:] == 0x11) and torch.all(ss[n_out:] == 7.0)
+
+
+def test_dispatch_fp8_backward_is_the_gather_sum(gpu):
+    """Autograd of the fused dispatch: straight through the quantiser, then d_tokens[t] = sum_j d_x_sorted[inv[t*k+j]]
+    (the backward of expand + permute), equal to the three-pass form's gradient bit for bit."""
+    from picotron_amd import _ops
+    from picotron_amd.expert_parallel import ep_communications as C
+
+    T, H, E, k = 96, 512, 8, 2
+    x = _c2_input(T, H, seed=5).bfloat16()
+    idx = torch.stack([torch.randperm(E, generator=torch.Generator().manual_seed(i))[:k] for i in range(T)])
+    plan = _ops.permute_plan(idx.reshape(-1).to(gpu), E)
+    up = torch.randn(T * k, H, generator=torch.Generator().manual_seed(6)).bfloat16().to(gpu)
+    a = x.to(gpu).requires_grad_(True)
+    ya, qa, sa = _ops.dispatch_fp8(a, plan.inv_order, k, T * k, with_codes=True)
+    assert qa.dtype == torch.uint8 and sa.dtype == torch.float32 and not qa.requires_grad
+    ya.backward(up)
+    b = x.to(gpu).requires_grad_(True)
+    yb = _ops.expand_permute(C.fp8_round_trip(b), plan.order, plan.inv_order, k, T * k)
+    yb.backward(up)
+    assert torch.equal(ya, yb) and torch.equal(a.grad, b.grad)
