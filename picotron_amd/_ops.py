@@ -34,8 +34,10 @@ class _Route(torch.autograd.Function):
         probs = _empty((T, E), torch.float32, dev)
         counts = partial = None
         n_part = 0
+        # one zero fill serves the pick counters (added to with integer atomics) and the aux-loss scalar
+        zeros = torch.zeros(E + 1 if balance else 1, dtype=torch.int32, device=dev)
         if balance:
-            counts = torch.zeros(E, dtype=torch.int32, device=dev)
+            counts = zeros[:E]
             if aux_coef > 0:
                 n_part = lib.picomoe_route_partials(T, E)
                 partial = _empty((n_part, E), torch.float32, dev)
@@ -46,7 +48,7 @@ class _Route(torch.autograd.Function):
             ),
             "picomoe_route_fwd",
         )
-        aux = torch.zeros((), dtype=torch.float32, device=dev)
+        aux = zeros[-1:].view(torch.float32).reshape(())
         if balance and T > 0:
             _lib.check(
                 lib.picomoe_balance(
@@ -58,6 +60,7 @@ class _Route(torch.autograd.Function):
         ctx.save_for_backward(probs, idx, counts)
         ctx.cfg = (top_k, bool(norm_topk), float(aux_coef) if balance else 0.0, logits.dtype)
         ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)   # no zero tensors for the outputs nobody differentiated (the indices, an unused aux)
         return idx, w, aux
 
     @staticmethod

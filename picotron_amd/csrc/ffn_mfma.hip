@@ -266,9 +266,13 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     int64_t pf_step;      // bytes per k-tile
     {
         const bool pf_b = wave >= NW / 2;
-        const int q = (wave % (NW / 2)) * 64 + lane, half = q & 1;
+        const int q = (wave % (NW / 2)) * 64 + lane;
         const int si = pf_b ? tc.b_si : tc.a_si, sn = pf_b ? tc.b_sn : tc.a_sn;
-        int j = si + sn * (q >> 1);  // line of the 256-line slice
+        // two touches (one per 64 bytes) of every sn-th line; a tile that shares its slice with nobody (a light tail, an
+        // expert of one row tile) touches every line once instead: at two touches per line its 256 lanes would only
+        // reach lines 0..127 and leave the other half of the slice to the demand loads
+        const int half = sn > 1 ? (q & 1) : 0;
+        int j = sn > 1 ? si + sn * (q >> 1) : q;  // line of the 256-line slice
         if (j >= 256) j = si;
         // X-major slices: line j is 128 bytes of k row j / 4; a segment shorter than one k-tile clamps the row
         int kr = j >> 2;
@@ -341,10 +345,14 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     };
     auto issue_a = [&](int kt, int stage, int q) { issue_a_at(a_tile(kt), kt == n_kt - 1, stage, q); };
     auto issue_b = [&](int kt, int stage, int q) { issue_b_at(b_tile(kt), kt == n_kt - 1, stage, q); };
+    // A wave whose 128 rows all lie past the segment (rows 128..255 of a tile of at most 128 rows) also fills tile rows
+    // nobody reads: its A loads are left out, in the prologue here and in its copy of the k-loop (a quarter of the loads
+    // of a light tile; 3 % of the gate/up launch at 64 skewed experts, nothing where light tiles are few).
+    const bool skip_a = MODE != kWgrad && active_blocks == 0;
     auto issue_tile = [&](int kt, int stage) {
 #pragma unroll
         for (int q = 0; q < QN; ++q) {
-            issue_a(kt, stage, q);
+            if (!skip_a) issue_a(kt, stage, q);
             issue_b(kt, stage, q);
         }
     };
@@ -531,6 +539,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             // vmcnt(2*QN): tile 0 has landed, tile 1 may still be in flight
             static_assert(QN == 4 || QN == 8, "wait counts below are written for 4 or 8 loads per operand, wave and k-tile");
             if (QN == 8) __builtin_amdgcn_s_waitcnt(0x4F70);
+            else if (skip_a) __builtin_amdgcn_s_waitcnt(0x0F74);  // only the B loads were issued: QN per tile
             else __builtin_amdgcn_s_waitcnt(0x0F78);
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -593,8 +602,12 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
                     if (kk < 2 && (n & ((1 << kSlotShift) - 1)) == 0) {
                         const int m = n >> kSlotShift;             // 0 .. 3
                         const int q = (QN / 2) * kk + (m >> 1);    // m = 0, 1: loads q of A and B; m = 2, 3: loads q + 1
-                        if ((m & 1) == 0) issue_a_at(a_next, next_is_last, stage ^ 1, q);
-                        else issue_b_at(b_next, next_is_last, stage ^ 1, q);
+                        constexpr bool kSkipA = MODE != kWgrad && decltype(active)::value == 0;
+                        if ((m & 1) == 0) {
+                            if (!kSkipA) issue_a_at(a_next, next_is_last, stage ^ 1, q);
+                        } else {
+                            issue_b_at(b_next, next_is_last, stage ^ 1, q);
+                        }
                     }
                     if (kk == 2 && n == (kWide ? 1 : 2)) prefetch_l2(kt);
                 });

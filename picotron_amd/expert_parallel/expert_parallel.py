@@ -30,6 +30,19 @@ def _argsort_inv(key, num_keys=None):
     return plan.order.to(torch.int64), plan.inv_order.to(torch.int64)
 
 
+_side_streams = {}
+
+
+def _side_stream(device):
+    """One extra stream per device (default priority), created on first use and shared by every layer: the layers of a
+    model run one after the other, so their shared experts never compete for it."""
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    stream = _side_streams.get(key)
+    if stream is None:
+        stream = _side_streams[key] = torch.cuda.Stream(device=key)
+    return stream
+
+
 class _StackedWeights(torch.autograd.Function):
     """Presents E per-expert parameters as one [E, ...] tensor without copying: ``stack`` already shares
     storage with them.  Backward hands each parameter its slice of the stacked gradient."""
@@ -75,6 +88,7 @@ class MoELayer(nn.Module):
         else:
             self.shared_expert = None
 
+        # ep_overlap: the shared expert runs on a second stream beside the routed path (see _shared_start); the other
         # knobs of the multi-rank paths are kept as attributes (callers set them) but have no effect here
         self.ep_overlap = getattr(config, "ep_overlap", True)
         self.ep_num_tiles = getattr(config, "ep_num_tiles", 1)
@@ -185,14 +199,33 @@ class MoELayer(nn.Module):
         return self.down_proj_latent(tokens) if self.latent else tokens
 
     def _shared_start(self, tokens):
+        """Starts the shared expert.  With ``ep_overlap`` it is enqueued on a second HIP stream (default priority), so its
+        kernels run beside the routed path's: at small batches neither the shared expert's launches (one expert: few
+        tiles) nor the routed ones fill the 256 CUs alone.  The reference overlaps the shared expert with the dispatch
+        exchange the same way (expert_parallel.py:230-248); autograd replays each backward op on the stream its forward
+        ran on, so the backward overlaps too."""
         if self.shared_expert is None:
             return None, None
-        return self.shared_expert(tokens), None
+        if not (self.ep_overlap and tokens.is_cuda):
+            return self.shared_expert(tokens), None
+        main = torch.cuda.current_stream(tokens.device)
+        side = _side_stream(tokens.device)
+        side.wait_stream(main)                   # tokens are ready once the work already queued on this stream is done
+        with torch.cuda.stream(side):
+            out = self.shared_expert(tokens)
+        tokens.record_stream(side)               # the allocator must not hand tokens' memory out before the side stream is done
+        return out, side
 
     def _finalize(self, y_expert, shared):
         y = self.up_proj_latent(y_expert) if self.latent else y_expert
-        shared_out, _ = shared
-        return y if shared_out is None else y + shared_out
+        shared_out, side = shared
+        if shared_out is None:
+            return y
+        if side is not None:
+            main = torch.cuda.current_stream(y.device)
+            main.wait_stream(side)
+            shared_out.record_stream(main)
+        return y + shared_out
 
     def _moe_naive(self, tokens, topk_idx, topk_weights):
         _lib.require_cuda(tokens, topk_idx, topk_weights)
