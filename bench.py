@@ -360,10 +360,26 @@ def mfma_ceiling(device, launches=8):
         flop = lib.picomoe_diag_mfma_loop_flop(shape, iters, n_blocks)
 
         def launch():
-            _lib.check(lib.picomoe_diag_mfma_loop(_lib.ptr(data), nbytes, shape, iters, n_blocks, None, st), "picomoe_diag_mfma_loop")
+            _lib.check(lib.picomoe_diag_mfma_loop(_lib.ptr(data), nbytes, shape, iters, 0, 0, n_blocks, None, st), "picomoe_diag_mfma_loop")
 
         ms = time_events(launch, launches, warm=3)
         out[name] = flop / ms / 1e9
+    # What a pause is worth: bursts of 40 iterations (about 40 us, the length of a k-loop of some 25 k-steps) with every
+    # block idle for 5 / 10 / 20 us between them.  If the power limit alone set the pace the average rate would not move
+    # (the clock would rise to use the budget the pause saves); if the clock did not react it would fall by the idle share.
+    nbytes, iters, burst = rand16.numel() * 2, 4800, 40
+    flop = lib.picomoe_diag_mfma_loop_flop(0, iters, n_blocks)
+    duty = {}
+    for idle_us in (5, 10, 20):
+        def launch():
+            _lib.check(lib.picomoe_diag_mfma_loop(_lib.ptr(rand16), nbytes, 0, iters, burst, idle_us, n_blocks, None, st), "picomoe_diag_mfma_loop")
+
+        ms = time_events(launch, launches, warm=3)
+        busy_ms = ms - (iters // burst) * idle_us * 1e-3
+        duty[f"idle_{idle_us}us_per_40_iterations"] = {
+            "average_tflops": flop / ms / 1e9, "tflops_inside_bursts": flop / busy_ms / 1e9, "idle_share": 1.0 - busy_ms / ms,
+            "share_of_the_idle_time_won_back": 1.0 - (1.0 - flop / ms / 1e9 / out["bf16_16x16x32"]) / (1.0 - busy_ms / ms)}
+    out["bursts_bf16_16x16x32"] = duty
     return out, n_blocks
 
 
@@ -720,7 +736,7 @@ def main():
             "hipblaslt_dense": {**dense, "what": "torch.nn.functional.linear (hipBLASLt), one dense GEMM over all routed rows "
                                                  "against one expert's weight matrix: x @ [gate_w; up_w].T and act @ down_w.T"},
         })
-        log(f"[bench] MFMA-only loop under the power limit: " + ", ".join(f"{k} {v:.0f}" for k, v in ceiling.items())
+        log(f"[bench] MFMA-only loop under the power limit: " + ", ".join(f"{k} {v:.0f}" for k, v in ceiling.items() if not isinstance(v, dict))
             + f" TFLOP/s; hipBLASLt dense gate_up {dense['gate_up']:.0f}, down {dense['down']:.0f} TFLOP/s")
         qg, dg, tq, td = fp8_quant_bandwidth(device)
         result["fp8_quant"] = {"GBps": qg, "frac_hbm": qg / HBM_PEAK_GBPS, "us": tq, "dequant_GBps": dg,

@@ -210,14 +210,17 @@ int picomoe_ffn_wgrad(const void* lhs, int64_t ld_lhs, const void* rhs, int64_t 
  * datasheet peak.  n_blocks blocks of 8 wavefronts (one block per CU fills the chip with two wavefronts per SIMD), each
  * wavefront multiplying the same operand fragments into 32 independent accumulator blocks `iters` times.  The fragments
  * are read once from `operands` (operand_bytes >= 16, 16-byte aligned; indices wrap), so the caller chooses the bit
- * patterns: random values draw more power than zeros.  `sink` may be NULL.
+ * patterns: random values draw more power than zeros.  `sink` may be NULL.  burst_iters > 0 (a divisor of iters) makes
+ * every block pause for idle_us (<= 1000) after each burst_iters iterations, all its wavefronts together: the rate inside
+ * the bursts against the rate of the uninterrupted loop says how much of a pause comes back as a higher clock, i.e. what
+ * a phase without MFMAs costs a kernel whose clock the power limit sets.  burst_iters == 0: no pauses.
  * picomoe_diag_mfma_loop_flop returns the FLOP one such launch performs (-1 for an unknown shape). */
 #define PICOMOE_DIAG_BF16_16X16X32 0 /* v_mfma_f32_16x16x32_bf16 */
 #define PICOMOE_DIAG_BF16_32X32X16 1 /* v_mfma_f32_32x32x16_bf16 */
 #define PICOMOE_DIAG_FP8_16X16X128 2 /* v_mfma_f32_16x16x128_f8f6f4 on E4M3 codes */
 int64_t picomoe_diag_mfma_loop_flop(int shape, int64_t iters, int n_blocks);
-int picomoe_diag_mfma_loop(const void* operands, int64_t operand_bytes, int shape, int64_t iters, int n_blocks, float* sink,
-                           void* stream);
+int picomoe_diag_mfma_loop(const void* operands, int64_t operand_bytes, int shape, int64_t iters, int64_t burst_iters,
+                           int64_t idle_us, int n_blocks, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -48,7 +48,7 @@ _SIGNATURES = {
     "picomoe_ffn_kernel_family": [_i32, _i64, _i64],
     "picomoe_ffn_wgrad": [_p, _i64, _p, _i64, _p, _i32, _i64, _i64, _i64, _i32, _p, _p],
     "picomoe_diag_mfma_loop_flop": [_i32, _i64, _i32],
-    "picomoe_diag_mfma_loop": [_p, _i64, _i32, _i64, _i32, _p, _p],
+    "picomoe_diag_mfma_loop": [_p, _i64, _i32, _i64, _i64, _i64, _i32, _p, _p],
 }
 _RESTYPES = {"picomoe_error_string": ctypes.c_char_p, "picomoe_permute_workspace_bytes": ctypes.c_int64,
              "picomoe_permute_plan_static_max_bytes": ctypes.c_int64,

@@ -49,6 +49,15 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.picomoe_ffn_dgrad_x(null, counts, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 0
     assert lib.picomoe_ffn_down(null, counts, 4, 8, 256, 128, null, null, 1, null, null, 0, null) == 1    # null tensors
     assert lib.picomoe_ffn_down(null, null, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 1      # null counts
+    # diagnostics and queries
+    assert lib.picomoe_diag_mfma_loop_flop(0, 10, 2) == 64 * 2 * 16 * 16 * 32 * 8 * 10 * 2
+    assert lib.picomoe_diag_mfma_loop_flop(9, 10, 2) == -1
+    assert lib.picomoe_diag_mfma_loop(null, 1024, 0, 10, 0, 0, 1, null, null) == 1                         # null operands
+    assert lib.picomoe_dispatch_fp8(null, 1, 0, 64, null, 2, 0, null, null, null, null, null, null) == 0   # no tokens
+    assert lib.picomoe_dispatch_fp8(null, 1, 4, 64, null, 17, 8, null, null, null, null, null, null) == 1  # top_k > 16
+    assert lib.picomoe_dispatch_fp8(null, 1, 4, 64, null, 2, 8, null, counts, null, null, null, null) == 1 # codes without scales
+    assert lib.picomoe_ffn_kernel_family(1, 4096, 14336) == 1 and lib.picomoe_ffn_kernel_family(0, 256, 512) == 2
+    assert lib.picomoe_ffn_kernel_family(1, 100, 36) == 0 and lib.picomoe_ffn_kernel_family(0, 16, 32) == 0
     with pytest.raises(_lib.PicomoeError):
         _lib.check(1, "demo")
 
