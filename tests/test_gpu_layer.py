@@ -550,3 +550,36 @@ def test_training_steps_follow_the_oracle(gpu):
     fresh.eval(); blocks[0].eval()
     with torch.no_grad():
         assert torch.equal(fresh(x.cuda()), blocks[0](x.cuda()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_shared_expert_on_a_second_stream_changes_nothing(gpu, dtype):
+    """``ep_overlap`` runs the shared expert on a second stream beside the routed path where the launches leave CUs idle
+    (every shape of this size): outputs and every gradient must equal, bit for bit, the run on one stream, for two
+    steps in a row (the second reuses memory the first released on either stream) and with work queued on the launch
+    stream right behind the layer."""
+    cfg = make_config(hidden=256, inter=128, num_experts=4, top_k=2, n_shared=1)
+    moe = build(cfg, seed=3, std=0.05, dtype=dtype)
+    assert moe._launches_leave_cus_idle(200) and not moe._launches_leave_cus_idle(10 ** 6)
+    g = torch.Generator().manual_seed(4)
+    xs = [torch.randn(2, 100, 256, generator=g).to(dtype) for _ in range(2)]
+    ups = [torch.randn(2, 100, 256, generator=g).to(dtype) for _ in range(2)]
+
+    def run(overlap):
+        moe.ep_overlap = overlap
+        results = []
+        for x, up in zip(xs, ups):
+            moe.zero_grad(set_to_none=True)
+            xin = x.cuda().requires_grad_(True)
+            out = moe(xin)
+            tail = out * 2.0 + 1.0                      # consumer queued on the launch stream right behind the layer
+            out.backward(up.cuda())
+            results.append([tail.detach().clone(), xin.grad.clone()] + [p.grad.clone() for p in moe.parameters()])
+        torch.cuda.synchronize()
+        return results
+
+    serial, overlapped = run(False), run(True)
+    for step_s, step_o in zip(serial, overlapped):
+        assert len(step_s) == len(step_o)
+        for a, b in zip(step_s, step_o):
+            assert torch.equal(a, b)
