@@ -150,7 +150,7 @@ int picomoe_combine_bwd(const void* d_out, const void* y, const int32_t* inv_ord
  * (optional) receives [g | u] for the backward pass. */
 int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                         int64_t inter, const void* gate_w, const void* up_w, int dtype, void* act, void* inter13,
-                        void* stream);
+                        void* workspace, int64_t workspace_bytes, void* stream);
 /* The same gate||up GEMM + silu_and_mul on FP8 MFMA, fed by the FP8 dispatch: xq [n_rows, hidden] E4M3 codes with one
  * fp32 scale per row (what _per_token_quant_fp8 ships, EP/ep_communications.py:63-68, instead of the dequantised rows
  * of :100), gate_wq / up_wq [E, inter, hidden] codes with one fp32 scale per output row ([E * inter], quantised the
@@ -176,17 +176,18 @@ int picomoe_ffn_down_fp8(const void* actq, const float* act_scale, const int64_t
  * d_inter13 [n_rows, 2*inter] = [dg | du]; act_out (optional) = silu(g) * u rebuilt from inter13. */
 int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                           int64_t inter, const void* down_w, const void* inter13, int dtype, void* d_inter13, void* act_out,
-                          void* stream);
+                          void* workspace, int64_t workspace_bytes, void* stream);
 /* Replaces dx = d_inter13 @ w13[e] (EP/megakernel.py:346) without the concatenated w13. */
 int picomoe_ffn_dgrad_x(const void* d_inter13, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                         int64_t inter, const void* gate_w, const void* up_w, int dtype, void* dx, void* workspace,
                         int64_t workspace_bytes, void* stream);
-/* Device scratch the two calls above can use (the library allocates nothing itself, the boundary rule of the reference's
- * kernels being torch-owned memory: EP/megakernel.py:294-306 allocates every buffer with torch.empty).  With
- * `workspace` of at least this many bytes the bf16 kernels cut the tiles of the last, partly filled round of blocks into
- * 2 or 4 ranges of K that run side by side, park the fp32 partial tiles there and add them up in a second small kernel;
- * with NULL (or fewer bytes) every tile is computed whole.  Results agree to the rounding of the fp32 partial sums.
- * Calls that overlap in time on different streams need a workspace each. */
+/* Device scratch the four row-grouped calls above (gate_up, down, dgrad_act, dgrad_x) can use (the library allocates nothing
+ * itself, the boundary rule of the reference's kernels being torch-owned memory: EP/megakernel.py:294-306 allocates every buffer
+ * with torch.empty).  With `workspace` of at least this many bytes the bf16 kernels cut the tiles of the last, partly filled
+ * round of blocks into 2 or 4 ranges of K that run side by side, park the fp32 partial tiles there and add them up in a second
+ * small kernel, which also applies the epilogue (SwiGLU, SwiGLU backward, row weight); with NULL (or fewer bytes) every tile is
+ * computed whole.  Results agree to the rounding of the fp32 partial sums.  Calls that overlap in time on different streams need
+ * a workspace each; calls of one stream can share one. */
 int64_t picomoe_ffn_workspace_bytes(void);
 /* Which kernels the five expert-FFN entry points run for a dtype and layer widths (a query, no launch):
  * PICOMOE_FFN_BF16_MFMA -- bf16, hidden and inter multiples of 64 and >= 128: 256 x 256 tiles on v_mfma_f32_16x16x32_bf16;

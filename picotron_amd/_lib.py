@@ -38,11 +38,11 @@ _SIGNATURES = {
     "picomoe_gather_rows": [_p, _p, _i32, _i64, _i64, _i32, _p, _p],
     "picomoe_combine_fwd": [_p, _p, _p, _i64, _i32, _i64, _i32, _p, _p],
     "picomoe_combine_bwd": [_p, _p, _p, _p, _i64, _i32, _i64, _i32, _p, _p, _p],
-    "picomoe_ffn_gate_up": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
+    "picomoe_ffn_gate_up": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p, _i64, _p],
     "picomoe_ffn_gate_up_fp8": [_p, _p, _p, _i32, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
     "picomoe_ffn_down_fp8": [_p, _p, _p, _i32, _i64, _i64, _i64, _p, _p, _p, _p, _p],
     "picomoe_ffn_down": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _i64, _p],
-    "picomoe_ffn_dgrad_act": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p],
+    "picomoe_ffn_dgrad_act": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _p, _i64, _p],
     "picomoe_ffn_dgrad_x": [_p, _p, _i32, _i64, _i64, _i64, _p, _p, _i32, _p, _p, _i64, _p],
     "picomoe_ffn_workspace_bytes": [],
     "picomoe_ffn_kernel_family": [_i32, _i64, _i64],

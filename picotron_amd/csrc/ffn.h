@@ -32,11 +32,11 @@ int ffn_simple_wgrad(const FfnShape& s, const void* lhs, int64_t ld_lhs, const v
 bool ffn_mfma_supported(const FfnShape& s);
 bool ffn_mfma_wgrad_supported(int dtype, int64_t P, int64_t Q, int64_t ld_lhs, int64_t ld_rhs, const void* lhs, const void* rhs);
 int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
-                     hipStream_t st);
+                     void* ws, int64_t ws_bytes, hipStream_t st);
 int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const void* row_weight, void* y, void* ws,
                   int64_t ws_bytes, hipStream_t st);
 int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, const void* inter13, void* d_inter13,
-                       void* act_out, hipStream_t st);
+                       void* act_out, void* ws, int64_t ws_bytes, hipStream_t st);
 int ffn_mfma_dgrad_x(const FfnShape& s, const void* d_inter13, const void* gate_w, const void* up_w, void* dx, void* ws,
                      int64_t ws_bytes, hipStream_t st);
 int64_t ffn_mfma_workspace_bytes();

@@ -13,12 +13,12 @@ bool fill_shape(FfnShape* s, const int64_t* counts, int E, int64_t n_rows, int64
 
 extern "C" int picomoe_ffn_gate_up(const void* x, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                                    int64_t inter, const void* gate_w, const void* up_w, int dtype, void* act, void* inter13,
-                                   void* stream) {
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
     FfnShape s;
     PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(x && gate_w && up_w && act);
-    if (ffn_mfma_supported(s)) return ffn_mfma_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
+    if (ffn_mfma_supported(s)) return ffn_mfma_gate_up(s, x, gate_w, up_w, act, inter13, workspace, workspace_bytes, (hipStream_t)stream);
     if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
     return ffn_simple_gate_up(s, x, gate_w, up_w, act, inter13, (hipStream_t)stream);
 }
@@ -70,12 +70,12 @@ extern "C" int picomoe_ffn_down(const void* act, const int64_t* counts, int num_
 
 extern "C" int picomoe_ffn_dgrad_act(const void* dy, const int64_t* counts, int num_experts, int64_t n_rows, int64_t hidden,
                                      int64_t inter, const void* down_w, const void* inter13, int dtype, void* d_inter13,
-                                     void* act_out, void* stream) {
+                                     void* act_out, void* workspace, int64_t workspace_bytes, void* stream) {
     FfnShape s;
     PICOMOE_CHECK_ARG(fill_shape(&s, counts, num_experts, n_rows, hidden, inter, dtype));
     if (n_rows == 0) return PICOMOE_OK;
     PICOMOE_CHECK_ARG(dy && down_w && inter13 && d_inter13);
-    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
+    if (ffn_mfma_supported(s)) return ffn_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, workspace, workspace_bytes, (hipStream_t)stream);
     if (ffn_f32_mfma_supported(s)) return ffn_f32_mfma_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
     return ffn_simple_dgrad_act(s, dy, down_w, inter13, d_inter13, act_out, (hipStream_t)stream);
 }

@@ -68,7 +68,7 @@ struct MfmaParams {
     int64_t ldo;
     uint16_t* out2;       // gate/up: inter13 (optional); dgrad_act: act_out (optional)
     const uint16_t* aux;  // down: row_weight; dgrad_act: inter13
-    float* ws;            // down, dgrad_x: fp32 partial tiles of the split last round (kSplitWorkspaceBytes), or null
+    float* ws;            // M-grouped modes: fp32 partial tiles of the split last round (kSplitWorkspaceBytes), or null
     int max_pieces;       // 1 = no split
 };
 
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     constexpr int RPW = QN * 8;         // K-major tile rows a wave fills
     constexpr int KPW = QN * 2;         // X-major k rows a wave fills
     __shared__ __attribute__((aligned(1024))) char lds[2 * kStageBytes];
-    constexpr bool kCanSplit = MODE == kDown || MODE == kDgradX;
+    constexpr bool kCanSplit = MODE != kWgrad;  // the M-grouped modes can cut the tiles of a partly filled last round along K
     TileCoord tc;
     if (MODE == kWgrad) {
         if (!locate_wgrad(p.counts, p.E, p.m_tiles, p.n_tiles, blockIdx.x / kNumXcd, &tc)) return;
@@ -810,10 +810,13 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 }
 
 // Second pass of a split last round: the blocks (b, y) add up the fp32 pieces of remainder tile b / 8 of XCD b % 8 (in
-// piece order, so the result does not depend on timing) and apply the epilogue of the unsplit kernel: accumulators
-// rounded to the output type; down: times the row weight, rounded again.  Block (b, y) takes rows 32y .. 32y + 31 of the
-// tile, eight per wavefront, and issues the loads of all its rows and pieces before it adds: one block per tile walking
-// its 256 rows took 20-75 us, the time of a load's latency per row.
+// piece order, so the result does not depend on timing) and apply the epilogue of the unsplit kernel to the sums:
+//   down, dgrad_x: rounded to the output type; down: times the row weight, rounded again;
+//   gate/up:       g and u rounded, act = silu(g) * u, [g | u] stored when asked for (the partial tile holds, per 64 columns
+//                  of a wave, 32 gate columns and then the 32 up columns of the same FFN columns: lane l + 8 holds the u of lane l's g);
+//   dgrad_act:     da rounded, then the SwiGLU backward at [g | u].
+// Block (b, y) takes rows 32y .. 32y + 31 of the tile, eight per wavefront, four columns per lane, and issues the loads of all
+// its rows and pieces before it adds: one block per tile walking its 256 rows took 20-75 us, the time of a load's latency per row.
 constexpr int kFixupRows = 32;
 template <int MODE>
 __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
@@ -823,8 +826,12 @@ __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
     TileCoord tc;
     if (!locate_tile_slot(p.counts, p.E, p.n_tiles, g, xcd, g.full + t, &tc)) return;
     const float* w = p.ws + (int64_t)(xcd * kCusPerXcd + t * g.pieces) * (BM * BN);
-    const int c4 = (threadIdx.x & 63) * 4;
-    if ((int64_t)tc.n_tile * BN + c4 >= p.N) return;  // columns past the output's last (N is a multiple of 8)
+    const int lane = threadIdx.x & 63;
+    const int c4 = lane * 4;  // column of the partial tile
+    // output column of the lane's four values, and whether it exists (N is a multiple of 8)
+    const int64_t out_col = MODE == kGateUp ? (int64_t)tc.n_tile * 128 + (lane >> 4) * 32 + (lane & 7) * 4 : (int64_t)tc.n_tile * BN + c4;
+    const bool col_ok = out_col < p.N;
+    if (MODE != kGateUp && !col_ok) return;  // (gate/up keeps every lane: the u values travel between lanes below)
     constexpr int kRowsPerWave = kFixupRows / 4;
     const int row0 = blockIdx.y * kFixupRows + (threadIdx.x >> 6) * kRowsPerWave;
     f32x4_t v[kRowsPerWave][kMaxSplit];
@@ -835,31 +842,78 @@ __global__ __launch_bounds__(256) void ffn_mfma_fixup_kernel(MfmaParams p) {
             const bool live = row0 + r < tc.rows && pc < g.pieces;
             v[r][pc] = live ? *(const f32x4_t*)(w + (int64_t)pc * (BM * BN) + (row0 + r) * BN + c4) : f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
+    auto round_bf16 = [](float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); };
+    auto store4 = [](uint16_t* dst, const float (&x)[4]) {
+        *(uint64_t*)dst = (uint64_t)pack_bf16x2(x[0], x[1]) | ((uint64_t)pack_bf16x2(x[2], x[3]) << 32);
+    };
+    auto load4 = [](const uint16_t* src, float (&x)[4]) {
+        const uint64_t bits = *(const uint64_t*)src;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = bf16_bits_to_f32((uint32_t)(bits >> (16 * i)) & 0xFFFFu);
+    };
 #pragma unroll
     for (int r = 0; r < kRowsPerWave; ++r) {
         const int row = row0 + r;
-        if (row >= tc.rows) break;
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        if (row >= tc.rows) break;  // wave-uniform
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int pc = 0; pc < kMaxSplit; ++pc) {  // pieces past g.pieces hold zeros: x + 0 leaves every sum as it is
-            s0 += v[r][pc][0]; s1 += v[r][pc][1]; s2 += v[r][pc][2]; s3 += v[r][pc][3];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] += v[r][pc][i];
         }
-        s0 = bf16_bits_to_f32(f32_to_bf16_bits(s0)); s1 = bf16_bits_to_f32(f32_to_bf16_bits(s1));
-        s2 = bf16_bits_to_f32(f32_to_bf16_bits(s2)); s3 = bf16_bits_to_f32(f32_to_bf16_bits(s3));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = round_bf16(s[i]);
         const int64_t grow = tc.row0 + row;
-        if (MODE == kDown && p.aux) {
-            const float rw = bf16_bits_to_f32(p.aux[grow]);
-            s0 *= rw; s1 *= rw; s2 *= rw; s3 *= rw;
+        if (MODE == kGateUp) {
+            const int64_t I = p.N;
+            float u[4], a[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) u[i] = __shfl(s[i], (lane + 8) & 63, 64);
+            if ((lane & 8) == 0 && col_ok) {  // the lanes that hold g
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[i] = round_bf16(s[i] * sigmoid_fast(s[i])) * u[i];
+                store4(p.out + grow * I + out_col, a);
+                if (p.out2) {
+                    store4(p.out2 + grow * 2 * I + out_col, s);
+                    store4(p.out2 + grow * 2 * I + I + out_col, u);
+                }
+            }
+        } else if (MODE == kDgradAct) {
+            const int64_t I = p.N;
+            float gv[4], uv[4], dg[4], du[4], a[4];
+            load4(p.aux + grow * 2 * I + out_col, gv);
+            load4(p.aux + grow * 2 * I + I + out_col, uv);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float sig = sigmoid_fast(gv[i]);
+                const float gs = gv[i] * sig;
+                dg[i] = s[i] * uv[i] * (sig + gs * (1.f - sig));
+                du[i] = s[i] * gs;
+                a[i] = round_bf16(gs) * uv[i];
+            }
+            store4(p.out + grow * 2 * I + out_col, dg);
+            store4(p.out + grow * 2 * I + I + out_col, du);
+            if (p.out2) store4(p.out2 + grow * I + out_col, a);
+        } else {
+            if (MODE == kDown && p.aux) {
+                const float rw = bf16_bits_to_f32(p.aux[grow]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[i] *= rw;
+            }
+            store4(p.out + grow * p.ldo + out_col, s);
         }
-        uint32_t o[2] = {pack_bf16x2(s0, s1), pack_bf16x2(s2, s3)};
-        *(uint64_t*)(p.out + grow * p.ldo + (int64_t)tc.n_tile * BN + c4) = (uint64_t)o[0] | ((uint64_t)o[1] << 32);
     }
 }
 
-// how many pieces the tiles of the last round may be cut into: none without the workspace, and none below 16 k-tiles a piece
-int split_pieces(const void* ws, int64_t ws_bytes, int64_t k_tiles) {
+// how many pieces the tiles of the last round may be cut into: none without the workspace, and none below 16 k-tiles a piece.
+// `rich_epilogue`: gate/up and dgrad_act, whose second pass redoes a SwiGLU epilogue over three (two) outputs per element and whose
+// pieces each park 256 KB of fp32 where the whole tile stores 192 KB of bf16: measured, the split pays for them from 64 k-tiles on
+// (hidden 4096: -1...2 % on ragged counts) and costs up to 20 % at 32 (hidden 2048, two pieces of 16 k-steps), so they split only
+// when four pieces are possible.
+int split_pieces(const void* ws, int64_t ws_bytes, int64_t k_tiles, bool rich_epilogue = false) {
     if (!ws || ws_bytes < kSplitWorkspaceBytes) return 1;
     const int64_t by_k = k_tiles / 16;
+    if (rich_epilogue) return by_k >= kMaxSplit ? kMaxSplit : 1;
     return by_k >= kMaxSplit ? kMaxSplit : (by_k >= 2 ? 2 : 1);
 }
 
@@ -883,13 +937,16 @@ bool ffn_mfma_supported(const FfnShape& s) {
 }
 
 int ffn_mfma_gate_up(const FfnShape& s, const void* x, const void* gate_w, const void* up_w, void* act, void* inter13,
-                     hipStream_t st) {
+                     void* ws, int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
     p.K = s.H; p.N = s.I; p.n_tiles = (int)((s.I + 127) / 128);
     p.A = (const uint16_t*)x; p.lda = s.H;
     p.B0 = (const uint16_t*)gate_w; p.B1 = (const uint16_t*)up_w; p.ldb = s.H; p.b_expert_stride = s.I * s.H;
     p.out = (uint16_t*)act; p.ldo = s.I; p.out2 = (uint16_t*)inter13;
-    hipLaunchKernelGGL((ffn_mfma_kernel<kGateUp, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
+    p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK, true);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kGateUp, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
+    if (p.max_pieces > 1)
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kGateUp>), dim3(kNumXcd * (kCusPerXcd / 2), BM / kFixupRows), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 
@@ -908,13 +965,16 @@ int ffn_mfma_down(const FfnShape& s, const void* act, const void* down_w, const 
 }
 
 int ffn_mfma_dgrad_act(const FfnShape& s, const void* dy, const void* down_w, const void* inter13, void* d_inter13,
-                       void* act_out, hipStream_t st) {
+                       void* act_out, void* ws, int64_t ws_bytes, hipStream_t st) {
     MfmaParams p = base_params(s);
     p.K = s.H; p.N = s.I; p.n_tiles = (int)((s.I + BN - 1) / BN);
     p.A = (const uint16_t*)dy; p.lda = s.H;
     p.B0 = (const uint16_t*)down_w; p.ldb = s.I; p.b_expert_stride = s.H * s.I;  // down_w[e] read as [K = H][N = I]
     p.out = (uint16_t*)d_inter13; p.ldo = 2 * s.I; p.out2 = (uint16_t*)act_out; p.aux = (const uint16_t*)inter13;
-    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradAct, kWaves>), dim3(grid_m_grouped(s, p.n_tiles)), dim3(kWaves * 64), 0, st, p);
+    p.ws = (float*)ws; p.max_pieces = split_pieces(ws, ws_bytes, p.K / BK, true);
+    hipLaunchKernelGGL((ffn_mfma_kernel<kDgradAct, kWaves>), dim3(grid_m_grouped(s, p.n_tiles, p.max_pieces > 1)), dim3(kWaves * 64), 0, st, p);
+    if (p.max_pieces > 1)
+        hipLaunchKernelGGL((ffn_mfma_fixup_kernel<kDgradAct>), dim3(kNumXcd * (kCusPerXcd / 2), BM / kFixupRows), dim3(256), 0, st, p);
     return picomoe_launch_status();
 }
 

@@ -67,9 +67,11 @@ def _gate_up(x, counts, gate_w, up_w, keep_inter13):
     N = x.shape[0]
     act = torch.empty((N, I), dtype=x.dtype, device=x.device)
     inter13 = torch.empty((N, 2 * I), dtype=x.dtype, device=x.device) if keep_inter13 else None
+    ws = _ffn_workspace(x.device) if x.dtype == torch.bfloat16 else None
     _lib.check(
         lib.picomoe_ffn_gate_up(_lib.ptr(x), _lib.ptr(counts), E, N, H, I, _lib.ptr(gate_w), _lib.ptr(up_w),
-                                _lib.dtype_code(x.dtype), _lib.ptr(act), _lib.ptr(inter13), _lib.stream_ptr()),
+                                _lib.dtype_code(x.dtype), _lib.ptr(act), _lib.ptr(inter13), _lib.ptr(ws),
+                                ws.numel() if ws is not None else 0, _lib.stream_ptr()),
         "picomoe_ffn_gate_up",
     )
     return act, inter13
@@ -146,7 +148,7 @@ _MAX_WORKSPACES = 4
 
 
 def _ffn_workspace(device):
-    """Scratch for the split last round of the down / dgrad_x kernels (picomoe_ffn_workspace_bytes, 64 MB): one buffer
+    """Scratch for the split last round of the row-grouped kernels (picomoe_ffn_workspace_bytes, 64 MB): one buffer
     per device and stream, allocated on first use -- kernels of one stream run one after the other, so they can share it.
     At most ``_MAX_WORKSPACES`` buffers are kept; when a further stream asks for one, the least recently used goes back
     to the caching allocator, which hands it out again only on the stream it was allocated and used on, i.e. in order
@@ -189,9 +191,11 @@ def _dgrad_act(dy, counts, down_w, inter13, want_act):
     N = dy.shape[0]
     d13 = torch.empty((N, 2 * I), dtype=dy.dtype, device=dy.device)
     act = torch.empty((N, I), dtype=dy.dtype, device=dy.device) if want_act else None
+    ws = _ffn_workspace(dy.device) if dy.dtype == torch.bfloat16 else None
     _lib.check(
         lib.picomoe_ffn_dgrad_act(_lib.ptr(dy), _lib.ptr(counts), E, N, H, I, _lib.ptr(down_w), _lib.ptr(inter13),
-                                  _lib.dtype_code(dy.dtype), _lib.ptr(d13), _lib.ptr(act), _lib.stream_ptr()),
+                                  _lib.dtype_code(dy.dtype), _lib.ptr(d13), _lib.ptr(act), _lib.ptr(ws),
+                                  ws.numel() if ws is not None else 0, _lib.stream_ptr()),
         "picomoe_ffn_dgrad_act",
     )
     return d13, act

@@ -193,6 +193,60 @@ def test_split_last_round_matches_whole_tiles(gpu, counts, H):
         assert torch.equal(fn(ws).float().cpu(), split)               # fixed summation order: run to run identical
 
 
+@pytest.mark.parametrize("H", [2048, 4096, 8192])
+@pytest.mark.parametrize("counts", [[300, 260, 100, 515], [256, 512, 7, 129], [40, 0, 3, 1]])
+def test_split_last_round_gate_up_and_dgrad_act(gpu, counts, H):
+    """The same split for the two kernels whose epilogue is more than a store: gate/up (SwiGLU on the summed pieces, [g | u]
+    kept) and dgrad_act (SwiGLU backward at [g | u] on the summed pieces, act rebuilt).  They split into four pieces from
+    K = hidden = 64 k-tiles on (4096, 8192 here) and not below (2048: the workspace changes nothing); FFN width 384 gives the
+    last tile column of dgrad_act only half its columns.  Whole-tile and split
+    results agree to the rounding of the partial sums, both with the oracle's arithmetic at the bf16 tolerance, run to run
+    identical, rows past the segments untouched."""
+    from picotron_amd import _lib
+
+    E, I = len(counts), 384
+    x, cnt, gw, uw, dw, g = _mk(E, H, I, counts, torch.bfloat16, 17, scale=0.02)
+    N, slack = x.shape[0], 5
+    dy = torch.randn(N, H, generator=g).bfloat16()
+    i13 = (torch.randn(N, 2 * I, generator=g) * 0.7).bfloat16()
+    pad = lambda t: torch.cat([t, torch.full((slack, t.shape[1]), float("nan"), dtype=t.dtype)]).cuda()
+    xd, dyd, i13d = pad(x), pad(dy), pad(i13)
+    cntd, gwd, uwd, dwd = cnt.cuda(), gw.cuda(), uw.cuda(), dw.cuda()
+    lib = _lib.load()
+    ws = torch.empty(lib.picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    P, code, st = _lib.ptr, _lib.dtype_code(torch.bfloat16), _lib.stream_ptr()
+    fill = lambda cols: torch.full((N + slack, cols), 7.0, dtype=torch.bfloat16, device="cuda")
+
+    def gate_up(workspace):
+        act, out13 = fill(I), fill(2 * I)
+        _lib.check(lib.picomoe_ffn_gate_up(P(xd), P(cntd), E, N + slack, H, I, P(gwd), P(uwd), code, P(act), P(out13), P(workspace),
+                                           workspace.numel() if workspace is not None else 0, st), "picomoe_ffn_gate_up")
+        return torch.cat([act, out13], 1)
+
+    def dgrad_act(workspace):
+        d13, act = fill(2 * I), fill(I)
+        _lib.check(lib.picomoe_ffn_dgrad_act(P(dyd), P(cntd), E, N + slack, H, I, P(dwd), P(i13d), code, P(d13), P(act), P(workspace),
+                                             workspace.numel() if workspace is not None else 0, st), "picomoe_ffn_dgrad_act")
+        return torch.cat([d13, act], 1)
+
+    owner = torch.repeat_interleave(torch.arange(E), cnt)
+    xf = x.float()
+    g13 = torch.cat([torch.einsum("nh,nih->ni", xf, gw.float()[owner]), torch.einsum("nh,nih->ni", xf, uw.float()[owner])], 1)
+    g13 = g13.bfloat16().float()
+    want_gu = torch.cat([torch.nn.functional.silu(g13[:, :I]).bfloat16().float() * g13[:, I:], g13], 1)
+    da = torch.einsum("nh,nhi->ni", dy.float(), dw.float()[owner]).bfloat16().float()
+    gi, ui = i13.float()[:, :I], i13.float()[:, I:]
+    want_da = torch.cat([O.silu_and_mul_bwd(i13.float(), da), torch.nn.functional.silu(gi).bfloat16().float() * ui], 1)
+    for fn, want in ((gate_up, want_gu), (dgrad_act, want_da)):
+        whole, split = fn(None).float().cpu(), fn(ws).float().cpu()
+        assert torch.all(whole[N:] == 7.0) and torch.all(split[N:] == 7.0)          # slack rows: untouched
+        whole, split = whole[:N], split[:N]
+        scale = want.abs().max()
+        assert (whole - want).abs().max() <= 1e-2 * scale and (split - want).abs().max() <= 1e-2 * scale
+        assert (split - whole).abs().max() <= 2.0 ** -6 * scale       # two bf16 roundings (g or da, then the product) of the largest value
+        assert torch.equal(fn(ws).float().cpu()[:N], split)           # fixed summation order: run to run identical
+
+
 @pytest.mark.parametrize("H,I,dtype", [(256, 384, torch.bfloat16), (320, 192, torch.bfloat16), (96, 40, torch.bfloat16), (96, 40, torch.float32),
                                        (18, 10, torch.float32)])
 def test_rows_past_the_segments_are_never_read_into_a_result(gpu, H, I, dtype):
@@ -220,12 +274,12 @@ def test_rows_past_the_segments_are_never_read_into_a_result(gpu, H, I, dtype):
         act, i13, y, d13, dx = fill(I), fill(2 * I), fill(H), fill(2 * I), fill(H)
         ws = torch.empty(lib.picomoe_ffn_workspace_bytes(), dtype=torch.uint8, device="cuda")
         P = _lib.ptr
-        _lib.check(lib.picomoe_ffn_gate_up(P(xs), P(cntd), E, N, H, I, P(gwd), P(uwd), code, P(act), P(i13), st), "gate_up")
+        _lib.check(lib.picomoe_ffn_gate_up(P(xs), P(cntd), E, N, H, I, P(gwd), P(uwd), code, P(act), P(i13), P(ws), ws.numel(), st), "gate_up")
         out_rows = {"act": act.clone(), "inter13": i13.clone()}
         # slack rows of the intermediates a later kernel reads: NaN, like the caller's torch.empty may hold
         act[n:], i13[n:] = float("nan"), float("nan")
         _lib.check(lib.picomoe_ffn_down(P(act), P(cntd), E, N, H, I, P(dwd), None, code, P(y), P(ws), ws.numel(), st), "down")
-        _lib.check(lib.picomoe_ffn_dgrad_act(P(dys), P(cntd), E, N, H, I, P(dwd), P(i13), code, P(d13), None, st), "dgrad_act")
+        _lib.check(lib.picomoe_ffn_dgrad_act(P(dys), P(cntd), E, N, H, I, P(dwd), P(i13), code, P(d13), None, P(ws), ws.numel(), st), "dgrad_act")
         out_rows.update(y=y.clone(), d13=d13.clone())
         d13[n:] = float("nan")
         _lib.check(lib.picomoe_ffn_dgrad_x(P(d13), P(cntd), E, N, H, I, P(gwd), P(uwd), code, P(dx), P(ws), ws.numel(), st), "dgrad_x")
