@@ -585,22 +585,44 @@ def train_step_bench(args):
         optimizer.step()
         return loss
 
+    timer = GemmTimer()
+    if not args.no_kernel_times:
+        timer.install()
     for _ in range(args.warmup):
         step()
+    if not args.no_kernel_times:
+        timer.prepare(2 * 60 * args.steps)   # 4 layers x (7 routed + 7 shared-expert launches) per step
     torch.cuda.synchronize()
+    if not args.no_kernel_times:
+        timer.start()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    timer.enabled = False
     n_params = sum(p.numel() for p in model.parameters())
     log(f"[bench] train_step: {ms:.3f} ms/step, {mbs * seq / ms * 1e3:,.0f} tokens/s, loss {float(loss.detach()):.3f}")
+    moe_gemms = None
+    if not args.no_kernel_times and timer.records:
+        # the expert GEMMs of the four MoE layers: 18 x rows x hidden x FFN FLOP for the routed rows and for the shared expert's
+        rows = mbs * seq
+        flop = 4 * 18.0 * (rows * cfg.num_experts_per_tok + rows * cfg.num_shared_experts) * cfg.hidden_size * cfg.intermediate_size
+        busy = timer.busy_ms() / args.steps
+        total = sum(st.elapsed_time(en) for _, _, st, en, _ in timer.records) / args.steps
+        moe_gemms = {"busy_ms_per_step": busy, "sum_of_launch_ms_per_step": total, "launches_per_step": len(timer.records) / args.steps,
+                     "flop_per_step": flop, "tflops": flop / busy / 1e9,
+                     "what": "grouped-GEMM launches of the 4 MoE layers (routed + shared expert); busy = time with at least one of them running"}
+        log(f"[bench] MoE expert GEMMs: {busy:.3f} ms/step busy ({total:.3f} ms summed over {len(timer.records) // args.steps} launches), "
+            f"{flop / busy / 1e9:.0f} TFLOP/s")
     print(json.dumps({
         "metric": "Llama-MoE train-step tokens/s (fwd + loss + bwd + AdamW, 1 GPU)", "value": mbs * seq / (ms * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "4-layer Llama, MoE feed-forward (hidden 2048, FFN 2048, 8 experts top-2 + 1 shared), "
-                               "seq 2048 x mbs 1, vocab 32000, fused AdamW", "tokens": mbs * seq, "parameters": n_params},
+                               "seq 2048 x mbs 1, vocab 32000, fused AdamW", "tokens": mbs * seq, "parameters": n_params,
+                   "shared_expert_on_second_stream": not args.no_shared_stream},
+        "moe_expert_gemms": moe_gemms,
     }), flush=True)
 
 
