@@ -569,7 +569,7 @@ def train_step_bench(args):
     model = Llama(cfg).to(torch.bfloat16).cuda().train()
     # fused=True: one pass over the 626 M parameters instead of the default implementation's seven (measured: 8.1 ms
     # of a 19.1 ms step went to the unfused update)
-    optimizer = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
+    optimizer = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True, capturable=args.hip_graph)
     torch.manual_seed(42)
     input_ids = torch.randint(0, cfg.vocab_size, (mbs, seq), device="cuda")
     target_ids = torch.randint(0, cfg.vocab_size, (mbs, seq), device="cuda")
@@ -584,6 +584,27 @@ def train_step_bench(args):
         loss.backward()
         optimizer.step()
         return loss
+
+    if args.hip_graph:
+        # The whole optimizer step as one HIP graph: at this size the step is a few hundred launches of 5-100 us each and
+        # the host cannot keep the GPU fed; captured once, a step is one graph launch.  (Nothing in the MoE layer
+        # synchronises with the host or allocates outside torch's allocator, so it captures as it is, second stream included.)
+        args.no_kernel_times = True          # events cannot be read out of a replayed graph
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        optimizer.zero_grad(set_to_none=True)
+        with torch.cuda.graph(graph):
+            static_loss = step()
+
+        def step():
+            graph.replay()
+            return static_loss
 
     timer = GemmTimer()
     if not args.no_kernel_times:
@@ -621,7 +642,7 @@ def train_step_bench(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "4-layer Llama, MoE feed-forward (hidden 2048, FFN 2048, 8 experts top-2 + 1 shared), "
                                "seq 2048 x mbs 1, vocab 32000, fused AdamW", "tokens": mbs * seq, "parameters": n_params,
-                   "shared_expert_on_second_stream": not args.no_shared_stream},
+                   "shared_expert_on_second_stream": not args.no_shared_stream, "hip_graph": bool(args.hip_graph)},
         "moe_expert_gemms": moe_gemms,
     }), flush=True)
 
@@ -636,6 +657,8 @@ def main():
     ap.add_argument("--no-kernel-times", action="store_true")
     ap.add_argument("--no-shared-stream", action="store_true",
                     help="run the shared expert on the launch stream, after the routed path's kernels instead of beside them")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="train_step only: capture the whole optimizer step (forward, loss, backward, AdamW) in one HIP graph and replay it")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="after the timed steps also launch a plain 1 GiB copy kernel three times: the known-size "
                          "reference that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
