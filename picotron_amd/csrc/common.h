@@ -35,8 +35,11 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return (uint32_t)__builtin_bit_cast(uint16_t, h);
 }
 
+// two fp32 -> two bf16 in one register (one v_cvt_pk_bf16_f32; round-to-nearest-even like f32_to_bf16_bits)
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 template <typename T>

@@ -504,6 +504,8 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         }
     };
     // The 16 MFMAs of phase kk with side(n) run after MFMA n (n = 0 .. 15): the slots for this wave's loads.
+    // The B fragment is the MFMA's first operand: the block comes out transposed, a lane holding four neighbouring
+    // columns of one output row (what the epilogue wants to convert and stage together).
     // `active` carries the number of 32-row blocks the wave computes; a wave without rows runs the side jobs alone.
     auto mma_with = [&](int kk, auto active, auto side) {
         if (kWide) {  // 8 MFMAs of 32 x 32 x 16, side(n) after MFMA n (n = 0 .. 7)
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
                 for (int j = 0; j < WJ; ++j) {
                     if (i < decltype(active)::value)
-                        accw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], accw[i][j], 0, 0, 0);
+                        accw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], accw[i][j], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                     side(i * WJ + j);
                     __builtin_amdgcn_sched_barrier(0);
@@ -525,7 +527,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
                 if (i < live_blocks(kk, decltype(active)::value))
-                    acc[4 * half + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[4 * half + i][j], 0, 0, 0);
+                    acc[4 * half + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[j], af[i], acc[4 * half + i][j], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 side(i * NJ + j);
                 __builtin_amdgcn_sched_barrier(0);
@@ -649,25 +651,29 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     __syncthreads();
 
     // ------------------------------------------------------------------------------------------
-    // epilogue.  A lane holds column (l & 15) and rows 4*(l >> 4) + r (r = 0..3) of each 16 x 16
-    // accumulator block: consecutive lanes are consecutive columns, 2 bytes apart in the output.  Each wave
-    // therefore stages 32 rows (two blocks) at a time through its own slice of LDS (the operand stages are free
-    // after the last barrier) and reads them back row-contiguously, so HBM sees 16-byte lanes and 128..256-byte
-    // row segments, and the fused SwiGLU backward reads g / u the same way.
+    // epilogue.  The MFMAs take the B fragment as their first operand, so an accumulator block is the transposed
+    // product: a lane holds row (l & 15) of each 16-row block and the four neighbouring columns 4*(l >> 4) .. +3 of each
+    // 16-column block (32 x 32 blocks: row (l & 31), columns 8q + 4*(l >> 5) .. +3, q = 0..3).  Four neighbours of an
+    // output row convert to bf16 two at a time and go to LDS as one 8-byte write.  Each wave stages 32 rows at a time
+    // through its own slice of LDS (the operand stages are free after the last barrier) and reads them back
+    // row-contiguously, so HBM sees 16-byte lanes and 128..256-byte row segments, and the fused SwiGLU backward reads
+    // g / u the same way.  The epilogues of gate/up and dgrad_act are bound by their vector instructions (some 130
+    // VALU cycles per element before this form), so what counts here is instructions per element: packed conversions,
+    // wave-uniform base pointers with one 32-bit lane offset, and a copy of every pass without bounds tests for the
+    // passes whose 32 rows and whose tile columns all exist.
     // ------------------------------------------------------------------------------------------
     if (kCanSplit && tc.pieces > 1) {
         // a piece of a split tile: the fp32 accumulators go to the workspace as they are; ffn_mfma_fixup_kernel adds the
         // pieces up in a fixed order and applies the epilogue
         float* w = p.ws + (int64_t)tc.ws_slot * (BM * BN);
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
+        for (int i = 0; i < NI; ++i) {
+            const int row = wm * 128 + i * 16 + l15;
+            if (row < tc.rows) {
 #pragma unroll
-            for (int j = 0; j < NJ; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = wm * 128 + i * 16 + g4 * 4 + r;
-                    if (row < tc.rows) w[row * BN + wn * CW + j * 16 + l15] = acc[i][j][r];
-                }
+                for (int j = 0; j < NJ; ++j) *(f32x4_t*)(w + row * BN + wn * CW + j * 16 + 4 * g4) = acc[i][j];
+            }
+        }
         return;
     }
     int valid_rows = tc.rows;
@@ -683,126 +689,195 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     constexpr int kChunksPerRow = kEpiCols / 8;
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
     static_assert(kReadIters >= 1, "a pass must cover at least one chunk per lane");
-
-    // value(b, j, r) -> float: 16-row block b (0, 1) of the 32 rows, j over the 16-column blocks of this pass, register r
-    auto stage_block = [&](auto value) {
+    constexpr int kRowsPerIt = 64 / kChunksPerRow;  // rows of a pass that one read-back iteration covers
+    // the 16-byte chunk this lane reads back and stores: row c_row + it * kRowsPerIt of the pass, columns c_col .. +7 of the
+    // wave's columns
+    const int c_row = lane / kChunksPerRow;
+    const int c_col = (lane % kChunksPerRow) * 8;
+    auto lo16 = [](uint32_t v) { return __uint_as_float(v << 16); };
+    auto hi16 = [](uint32_t v) { return __uint_as_float(v & 0xFFFF0000u); };
+    auto pack4 = [](const f32x4_t& v) { return u32x2_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])}; };
+    // packed(b, j) -> the four bf16 of 16-row block b (0, 1) of the pass and 16-column block j of the wave's pass columns
+    auto stage_block = [&](auto packed) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // earlier read-backs of this slice are done
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int j = 0; j < kEpiCols / 16; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = b * 16 + g4 * 4 + r;
-                    *(uint16_t*)(epi + row * kEpiStride + (j * 16 + l15) * 2) = (uint16_t)f32_to_bf16_bits(value(b, j, r));
-                }
+                *(u32x2_t*)(epi + (b * 16 + l15) * kEpiStride + (j * 16 + 4 * g4) * 2) = packed(b, j);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    // the same for a 32 x 32 block row: a lane holds column (l & 31) and rows 8*(r/4) + 4*(l >> 5) + (r % 4); value(j, r)
-    auto stage_block_wide = [&](auto value) {
+    // the same for a 32 x 32 block row; packed(j, q): 32-column block j, column group q
+    auto stage_block_wide = [&](auto packed) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int j = 0; j < kEpiCols / 32; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                *(uint16_t*)(epi + row * kEpiStride + (j * 32 + (lane & 31)) * 2) = (uint16_t)f32_to_bf16_bits(value(j, r));
-            }
+            for (int q = 0; q < 4; ++q)
+                *(u32x2_t*)(epi + (lane & 31) * kEpiStride + (j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = packed(j, q);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    // for_chunks(i, f): f(row_in_tile, col_in_wave_pass, 8 staged bf16 as u32x4)
-    auto for_chunks = [&](int i, auto f) {
-#pragma unroll
-        for (int it = 0; it < kReadIters; ++it) {
-            const int idx = it * 64 + lane;
-            const int row = idx / kChunksPerRow, ch = idx % kChunksPerRow;
-            const u32x4_t v = *(const u32x4_t*)(epi + row * kEpiStride + ch * 16);
-            const int trow = wm * 128 + i * 32 + row;
-            if (trow < valid_rows) f(trow, ch * 8, v);
-        }
+    auto read_chunk = [&](int it) { return *(const u32x4_t*)(epi + (it * kRowsPerIt + c_row) * kEpiStride + c_col * 2); };
+    // pass i (0..3) covers tile rows wm*128 + 32i .. +31
+    auto pass_live = [&](int i) { return wm * 128 + i * 32 < valid_rows; };  // wave-uniform
+    const bool cols_full = (int64_t)(tc.n_tile + 1) * (MODE == kGateUp ? BN / 2 : BN) <= p.N;
+    // f(std::true_type) when every row of pass i and every column of the tile exists, f(std::false_type) otherwise
+    auto with_fullness = [&](int i, auto f) {
+        if (cols_full && wm * 128 + i * 32 + 32 <= valid_rows) f(std::true_type{});
+        else f(std::false_type{});
     };
+    auto row_ok = [&](int i, int it) { return wm * 128 + i * 32 + it * kRowsPerIt + c_row < valid_rows; };
 
-    // i runs over the wave's four 32-row passes; pass i holds the accumulator blocks 2i and 2i + 1
     if (MODE == kGateUp) {
         const int64_t I = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
+        // (I is a multiple of 8: a 16-byte chunk lies inside the row or past its end as a whole)
+        const bool col_ok = col0 + c_col < I;
+        const uint32_t off_act = (uint32_t)((c_row * (int)I + c_col) * 2);      // the lane's chunk in iteration 0, bytes
+        const uint32_t off_gu = (uint32_t)((c_row * 2 * (int)I + c_col) * 2);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if (wm * 128 + i * 32 >= valid_rows) continue;  // wave-uniform: a block of rows past the segment has nothing to store
-            // g and u rounded to bf16 in place (what the reference's two Linear outputs hold)
+            if (!pass_live(i)) continue;  // wave-uniform: a block of rows past the segment has nothing to store
+            // g and u rounded to bf16 (what the reference's two Linear outputs hold), kept as packed pairs: column blocks
+            // 0, 1 of the wave hold g, blocks 2, 3 the u of the same output columns
+            u32x2_t gb[2][NJ / 2], ub[2][NJ / 2];
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
-                for (int j = 0; j < NJ; ++j)
+                for (int j = 0; j < NJ / 2; ++j) {
+                    gb[b][j] = pack4(acc[2 * i + b][j]);
+                    ub[b][j] = pack4(acc[2 * i + b][j + NJ / 2]);
+                }
+            stage_block([&](int b, int j) {
+                u32x2_t o;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[2 * i + b][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][j][r]));
-            // column blocks 0, 1 of the wave hold g, blocks 2, 3 the u of the same output columns
-            stage_block([&](int b, int j, int r) {
-                const float g = acc[2 * i + b][j][r], u = acc[2 * i + b][j + NJ / 2][r];
-                return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
+                for (int h = 0; h < 2; ++h) {
+                    const float g0 = lo16(gb[b][j][h]), g1 = hi16(gb[b][j][h]);
+                    const uint32_t s = pack_bf16x2(g0 * sigmoid_fast(g0), g1 * sigmoid_fast(g1));  // silu(g), rounded
+                    o[h] = pack_bf16x2(lo16(s) * lo16(ub[b][j][h]), hi16(s) * hi16(ub[b][j][h]));
+                }
+                return o;
             });
-            // (I is a multiple of 8: a 16-byte chunk lies inside the row or past its end as a whole)
-            for_chunks(i, [&](int trow, int c, u32x4_t v) {
-                if (col0 + c < I) *(u32x4_t*)(p.out + (out_row0 + trow) * I + col0 + c) = v;
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const int64_t r0 = out_row0 + wm * 128 + i * 32;
+                char* act_base = (char*)(p.out + r0 * I + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it)
+                    if (kFull || (row_ok(i, it) && col_ok))
+                        *(u32x4_t*)(act_base + (int64_t)it * kRowsPerIt * I * 2 + off_act) = read_chunk(it);
+                if (p.out2) {
+                    char* gu_base = (char*)(p.out2 + r0 * 2 * I + col0);
+                    stage_block([&](int b, int j) { return gb[b][j]; });
+#pragma unroll
+                    for (int it = 0; it < kReadIters; ++it)
+                        if (kFull || (row_ok(i, it) && col_ok))
+                            *(u32x4_t*)(gu_base + (int64_t)it * kRowsPerIt * I * 4 + off_gu) = read_chunk(it);
+                    stage_block([&](int b, int j) { return ub[b][j]; });
+#pragma unroll
+                    for (int it = 0; it < kReadIters; ++it)
+                        if (kFull || (row_ok(i, it) && col_ok))
+                            *(u32x4_t*)(gu_base + I * 2 + (int64_t)it * kRowsPerIt * I * 4 + off_gu) = read_chunk(it);
+                }
             });
-            if (p.out2) {
-                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) {
-                    if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + col0 + c) = v;
-                });
-                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j + NJ / 2][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) {
-                    if (col0 + c < I) *(u32x4_t*)(p.out2 + (out_row0 + trow) * 2 * I + I + col0 + c) = v;
-                });
-            }
         }
-    } else {
+    } else if (MODE == kDgradAct) {
+        const int64_t I = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
+        const bool col_ok = col0 + c_col < I;
+        const uint32_t off2 = (uint32_t)((c_row * 2 * (int)I + c_col) * 2);  // in the [.., 2I] tensors, bytes
+        const uint32_t off1 = (uint32_t)((c_row * (int)I + c_col) * 2);      // in act_out
+        const bool want_act = p.out2 != nullptr;  // the recomputed activation is only worked out when asked for
+        // the [g | u] chunks of a pass are loaded one pass ahead, into two register sets
+        u32x4_t gq[2][kReadIters], uq[2][kReadIters];
+        auto load_gu = [&](int i) {
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const char* base = (const char*)(p.aux + (out_row0 + wm * 128 + i * 32) * 2 * I + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it)
+                    if (kFull || (row_ok(i, it) && col_ok)) {
+                        gq[i & 1][it] = *(const u32x4_t*)(base + (int64_t)it * kRowsPerIt * I * 4 + off2);
+                        uq[i & 1][it] = *(const u32x4_t*)(base + I * 2 + (int64_t)it * kRowsPerIt * I * 4 + off2);
+                    }
+            });
+        };
+        if (pass_live(0)) load_gu(0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if (wm * 128 + i * 32 >= valid_rows) continue;
-            if (kWide) stage_block_wide([&](int j, int r) { return accw[i][j][r]; });
-            else stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) {
-                const int64_t col = col0 + c;
-                if (col >= p.N) return;
-                const int64_t grow = out_row0 + trow;
-                if (MODE == kDgradAct) {
-                    const int64_t I = p.N;
-                    const u32x4_t gv = *(const u32x4_t*)(p.aux + grow * 2 * I + col);
-                    const u32x4_t uv = *(const u32x4_t*)(p.aux + grow * 2 * I + I + col);
-                    u32x4_t dgv, duv, av;
-                    const bool want_act = p.out2 != nullptr;  // the recomputed activation is only worked out when asked for
+            if (!pass_live(i)) continue;
+            if (i + 1 < 4 && pass_live(i + 1)) load_gu(i + 1);
+            stage_block([&](int b, int j) { return pack4(acc[2 * i + b][j]); });  // da, rounded to bf16
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const int64_t r0 = out_row0 + wm * 128 + i * 32;
+                char* out_base = (char*)(p.out + r0 * 2 * I + col0);
+                char* act_base = (char*)(p.out2 + r0 * I + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it) {
+                    if (!(kFull || (row_ok(i, it) && col_ok))) continue;
+                    const u32x4_t v = read_chunk(it), gv = gq[i & 1][it], uv = uq[i & 1][it];
+                    u32x4_t dgv, duv;
+                    float gs8[8];  // silu(g), for the activation
 #pragma unroll
                     for (int w2 = 0; w2 < 4; ++w2) {
-                        float o_dg[2], o_du[2], o_a[2] = {0.f, 0.f};
+                        float o_dg[2], o_du[2];
 #pragma unroll
                         for (int h2 = 0; h2 < 2; ++h2) {
-                            const float da = __uint_as_float(h2 ? (v[w2] & 0xFFFF0000u) : (v[w2] << 16));
-                            const float g = __uint_as_float(h2 ? (gv[w2] & 0xFFFF0000u) : (gv[w2] << 16));
-                            const float u = __uint_as_float(h2 ? (uv[w2] & 0xFFFF0000u) : (uv[w2] << 16));
+                            const float da = h2 ? hi16(v[w2]) : lo16(v[w2]);
+                            const float g = h2 ? hi16(gv[w2]) : lo16(gv[w2]);
+                            const float u = h2 ? hi16(uv[w2]) : lo16(uv[w2]);
                             const float sig = sigmoid_fast(g);
                             const float gs = g * sig;
                             o_dg[h2] = da * u * (sig + gs * (1.f - sig));
                             o_du[h2] = da * gs;
-                            if (want_act) o_a[h2] = bf16_bits_to_f32(f32_to_bf16_bits(gs)) * u;
+                            gs8[2 * w2 + h2] = gs;
                         }
                         dgv[w2] = pack_bf16x2(o_dg[0], o_dg[1]);
                         duv[w2] = pack_bf16x2(o_du[0], o_du[1]);
-                        av[w2] = pack_bf16x2(o_a[0], o_a[1]);
                     }
-                    *(u32x4_t*)(p.out + grow * 2 * I + col) = dgv;
-                    *(u32x4_t*)(p.out + grow * 2 * I + I + col) = duv;
-                    if (want_act) *(u32x4_t*)(p.out2 + grow * I + col) = av;
-                } else if (MODE == kDown && p.aux) {
-                    const float rw = bf16_bits_to_f32(p.aux[grow]);
-                    u32x4_t o;
+                    *(u32x4_t*)(out_base + (int64_t)it * kRowsPerIt * I * 4 + off2) = dgv;
+                    *(u32x4_t*)(out_base + I * 2 + (int64_t)it * kRowsPerIt * I * 4 + off2) = duv;
+                    if (want_act) {  // one branch per chunk, after its stores
+                        u32x4_t av;
 #pragma unroll
-                    for (int w2 = 0; w2 < 4; ++w2)
-                        o[w2] = pack_bf16x2(__uint_as_float(v[w2] << 16) * rw, __uint_as_float(v[w2] & 0xFFFF0000u) * rw);
-                    *(u32x4_t*)(p.out + grow * p.ldo + col) = o;
-                } else {
-                    *(u32x4_t*)(p.out + grow * p.ldo + col) = v;
+                        for (int w2 = 0; w2 < 4; ++w2) {
+                            const uint32_t sl = pack_bf16x2(gs8[2 * w2], gs8[2 * w2 + 1]);  // silu(g), rounded
+                            av[w2] = pack_bf16x2(lo16(sl) * lo16(uv[w2]), hi16(sl) * hi16(uv[w2]));
+                        }
+                        *(u32x4_t*)(act_base + (int64_t)it * kRowsPerIt * I * 2 + off1) = av;
+                    }
+                }
+            });
+        }
+    } else {
+        const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
+        const bool col_ok = col0 + c_col < p.N;
+        const uint32_t off = (uint32_t)((c_row * (int)p.ldo + c_col) * 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (!pass_live(i)) continue;
+            if (kWide) {
+                stage_block_wide([&](int j, int q) {
+                    return u32x2_t{pack_bf16x2(accw[i][j][4 * q], accw[i][j][4 * q + 1]), pack_bf16x2(accw[i][j][4 * q + 2], accw[i][j][4 * q + 3])};
+                });
+            } else {
+                stage_block([&](int b, int j) { return pack4(acc[2 * i + b][j]); });
+            }
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const int64_t r0 = out_row0 + wm * 128 + i * 32;
+                char* out_base = (char*)(p.out + r0 * p.ldo + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it) {
+                    if (!(kFull || (row_ok(i, it) && col_ok))) continue;
+                    u32x4_t v = read_chunk(it);
+                    if (MODE == kDown && p.aux) {
+                        const float rw = bf16_bits_to_f32(p.aux[r0 + it * kRowsPerIt + c_row]);
+#pragma unroll
+                        for (int w2 = 0; w2 < 4; ++w2) v[w2] = pack_bf16x2(lo16(v[w2]) * rw, hi16(v[w2]) * rw);
+                    }
+                    *(u32x4_t*)(out_base + (int64_t)it * kRowsPerIt * p.ldo * 2 + off) = v;
                 }
             });
         }
