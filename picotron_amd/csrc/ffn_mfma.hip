@@ -85,36 +85,33 @@ __device__ __forceinline__ int swz_x(int kr) {
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 
-// Logical tile id of this block with the XCD remap, or -1.
-__device__ __forceinline__ int64_t logical_tile(int64_t total, int64_t slot) {
-    const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
-    if (slot >= per_xcd) return -1;
-    const int64_t L = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
-    return L < total ? L : -1;
-}
-
 // wgrad tiles: expert by expert; inside an expert the P x Q tile grid is walked in bands of 4 tile columns and, inside
 // a band, in groups of 8 tile rows (tile row fastest inside a group), so that any 32 consecutive tiles -- what one
 // XCD's 32 CUs run at a time -- form an 8 x 4 patch that needs only 8 + 4 operand slices per k-step from its L2.
-__device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, int64_t slot, TileCoord* tc) {
-    const int64_t per_e = (int64_t)m_tiles * n_tiles;
-    const int64_t L = logical_tile(per_e * E, slot);
-    if (L < 0) return false;
-    const int e = (int)(L / per_e);
-    const int rem = (int)(L % per_e);
-    constexpr int GM = 8, GN = 4;
-    const int band = rem / (m_tiles * GN), r = rem % (m_tiles * GN);
-    const int wn = n_tiles - band * GN < GN ? n_tiles - band * GN : GN;
-    const int g = r / (GM * wn), r2 = r % (GM * wn);
-    const int hm = m_tiles - g * GM < GM ? m_tiles - g * GM : GM;
-    tc->e = e;
-    tc->m_tile = g * GM + r2 % hm;
-    tc->n_tile = band * GN + r2 / hm;
-    tc->a_sn = wn;
-    tc->a_si = r2 / hm;
-    tc->b_sn = hm;
-    tc->b_si = r2 % hm;
-    tc->row0 = segment_start(counts, e);
+// (32-bit unsigned arithmetic throughout: see GroupedLayout.)
+__device__ __forceinline__ bool locate_wgrad(const int64_t* counts, int E, int m_tiles, int n_tiles, uint32_t slot, TileCoord* tc) {
+    const uint32_t per_e = (uint32_t)m_tiles * (uint32_t)n_tiles, total = per_e * (uint32_t)E;
+    // logical tile id of this block with the XCD remap
+    const uint32_t per_xcd = (total + kNumXcd - 1) / (uint32_t)kNumXcd;
+    if (slot >= per_xcd) return false;
+    const uint32_t L = (blockIdx.x % kNumXcd) * per_xcd + slot;
+    if (L >= total) return false;
+    const uint32_t e = L / per_e, rem = L - e * per_e;
+    constexpr uint32_t GM = 8, GN = 4;
+    const uint32_t um = (uint32_t)m_tiles, un = (uint32_t)n_tiles;
+    const uint32_t band = rem / (um * GN), r = rem - band * (um * GN);
+    const uint32_t wn = un - band * GN < GN ? un - band * GN : GN;
+    const uint32_t g = r / (GM * wn), r2 = r - g * (GM * wn);
+    const uint32_t hm = um - g * GM < GM ? um - g * GM : GM;
+    const uint32_t q = r2 / hm, rm = r2 - q * hm;
+    tc->e = (int)e;
+    tc->m_tile = (int)(g * GM + rm);
+    tc->n_tile = (int)(band * GN + q);
+    tc->a_sn = (int)wn;
+    tc->a_si = (int)q;
+    tc->b_sn = (int)hm;
+    tc->b_si = (int)rm;
+    tc->row0 = segment_start(counts, (int)e);
     tc->rows = uniform_i32((int)counts[e]);
     return true;
 }
@@ -147,9 +144,11 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int wm = wave / kWaveCols, wn = wave % kWaveCols;
     const int l15 = lane & 15, g4 = lane >> 4;
     // k-tiles of this block: all of K, or this piece's share of it
-    const int n_kt_all = MODE == kWgrad ? (tc.rows + BK - 1) / BK : (int)(p.K / BK);
-    const int kt_first = kCanSplit ? (int)((int64_t)tc.piece * n_kt_all / tc.pieces) : 0;
-    const int n_kt = kCanSplit ? (int)((int64_t)(tc.piece + 1) * n_kt_all / tc.pieces) - kt_first : n_kt_all;
+    const int n_kt_all = MODE == kWgrad ? (int)((uint32_t)(tc.rows + BK - 1) / BK) : (int)((uint64_t)p.K / BK);
+    // (pieces is 1, 2 or 4: the quotient is a shift)
+    const int pieces_lg = tc.pieces >> 1;
+    const int kt_first = kCanSplit ? (tc.piece * n_kt_all) >> pieces_lg : 0;
+    const int n_kt = kCanSplit ? (((tc.piece + 1) * n_kt_all) >> pieces_lg) - kt_first : n_kt_all;
     // a wavefront whose 128 rows all lie past the end of the expert's segment keeps loading and synchronising
     // but skips its fragment reads and MFMAs
     // 32-row blocks of this wave's 128 rows that hold rows of the expert's segment (wgrad: all four; its ragged dimension is K)
@@ -255,6 +254,47 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
             if (!T::kBKMajor) b_off_tail[q] = (uint32_t)((int)b_off[q] + dk * (int)p.ldb * 2);
         }
     }
+    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage.  The loads are the
+    // opaque form: every wait between a load and the LDS reads of its data is written out in this kernel (prologue,
+    // sub-step 3 of the k-loop, the end of the loop), the compiler adds none.
+    // ab / bb: the wave-uniform address of the operand's k-tile; last: it is the segment's last k-tile (wgrad's clamped offsets)
+    auto a_tile = [&](int kt) { return a_base + (int64_t)kt * a_step; };
+    auto b_tile = [&](int kt) { return b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0); };
+    auto issue_a_at = [&](const char* ab, bool last, int stage, int q) {
+        char* base = lds + stage * kStageBytes;
+        if (T::kAKMajor)
+            load16_to_lds_opaque(ab, a_off[q], base + (wave * RPW + q * 8) * 128);
+        else
+            load16_to_lds_opaque(ab, MODE == kWgrad && last ? a_off_tail[q] : a_off[q], base + (wave * KPW + q * 2) * 512);
+    };
+    auto issue_b_at = [&](const char* bb, bool last, int stage, int q) {
+        char* base = lds + stage * kStageBytes + kTileBytes;
+        if (T::kBKMajor)
+            load16_to_lds_opaque(bb, b_off[q], base + (wave * RPW + q * 8) * 128);
+        else
+            load16_to_lds_opaque(bb, MODE == kWgrad && last ? b_off_tail[q] : b_off[q], base + (wave * KPW + q * 2) * 512);
+    };
+    auto issue_a = [&](int kt, int stage, int q) { issue_a_at(a_tile(kt), kt == n_kt - 1, stage, q); };
+    auto issue_b = [&](int kt, int stage, int q) { issue_b_at(b_tile(kt), kt == n_kt - 1, stage, q); };
+    // A wave whose 128 rows all lie past the segment (rows 128..255 of a tile of at most 128 rows) also fills tile rows
+    // nobody reads: its A loads are left out, in the prologue here and in its copy of the k-loop (a quarter of the loads
+    // of a light tile; 3 % of the gate/up launch at 64 skewed experts, nothing where light tiles are few).
+    const bool skip_a = MODE != kWgrad && active_blocks == 0;
+    auto issue_tile = [&](int kt, int stage) {
+#pragma unroll
+        for (int q = 0; q < QN; ++q) {
+            if (!skip_a) issue_a(kt, stage, q);
+            issue_b(kt, stage, q);
+        }
+    };
+
+    // The first two k-tiles go out before anything else is set up (prefetch pointers, fragment addresses, the zeroed
+    // accumulators): what follows runs under their latency.
+    if (n_kt > 0) {
+        issue_tile(0, 0);
+        if (n_kt > 1) issue_tile(1, 1);
+    }
+
     // ------------------------------------------------------------------------------------------
     // L2 prefetch.  The demand loads of the blocks that share an operand slice reach the L2 together, and when the
     // slice still has to come from HBM they all queue behind the same misses.  So every k-step each wave touches
@@ -321,40 +361,6 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
         int64_t adv = kp < pf_n_kt ? pf_step : 0;
         if (MODE == kDgradX && kp == b_switch_kt) adv += pf_switch_delta;
         pf_cur += adv;
-    };
-
-    // one load instruction (q of QN) of this wave for the A or the B tile of k-tile kt into a stage.  The loads are the
-    // opaque form: every wait between a load and the LDS reads of its data is written out in this kernel (prologue,
-    // sub-step 3 of the k-loop, the end of the loop), the compiler adds none.
-    // ab / bb: the wave-uniform address of the operand's k-tile; last: it is the segment's last k-tile (wgrad's clamped offsets)
-    auto a_tile = [&](int kt) { return a_base + (int64_t)kt * a_step; };
-    auto b_tile = [&](int kt) { return b_base + (int64_t)kt * b_step + (kt >= b_switch_kt ? b_switch_delta : 0); };
-    auto issue_a_at = [&](const char* ab, bool last, int stage, int q) {
-        char* base = lds + stage * kStageBytes;
-        if (T::kAKMajor)
-            load16_to_lds_opaque(ab, a_off[q], base + (wave * RPW + q * 8) * 128);
-        else
-            load16_to_lds_opaque(ab, MODE == kWgrad && last ? a_off_tail[q] : a_off[q], base + (wave * KPW + q * 2) * 512);
-    };
-    auto issue_b_at = [&](const char* bb, bool last, int stage, int q) {
-        char* base = lds + stage * kStageBytes + kTileBytes;
-        if (T::kBKMajor)
-            load16_to_lds_opaque(bb, b_off[q], base + (wave * RPW + q * 8) * 128);
-        else
-            load16_to_lds_opaque(bb, MODE == kWgrad && last ? b_off_tail[q] : b_off[q], base + (wave * KPW + q * 2) * 512);
-    };
-    auto issue_a = [&](int kt, int stage, int q) { issue_a_at(a_tile(kt), kt == n_kt - 1, stage, q); };
-    auto issue_b = [&](int kt, int stage, int q) { issue_b_at(b_tile(kt), kt == n_kt - 1, stage, q); };
-    // A wave whose 128 rows all lie past the segment (rows 128..255 of a tile of at most 128 rows) also fills tile rows
-    // nobody reads: its A loads are left out, in the prologue here and in its copy of the k-loop (a quarter of the loads
-    // of a light tile; 3 % of the gate/up launch at 64 skewed experts, nothing where light tiles are few).
-    const bool skip_a = MODE != kWgrad && active_blocks == 0;
-    auto issue_tile = [&](int kt, int stage) {
-#pragma unroll
-        for (int q = 0; q < QN; ++q) {
-            if (!skip_a) issue_a(kt, stage, q);
-            issue_b(kt, stage, q);
-        }
     };
 
     // ------------------------------------------------------------------------------------------
@@ -535,9 +541,7 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     };
 
     if (n_kt > 0) {
-        issue_tile(0, 0);
         if (n_kt > 1) {
-            issue_tile(1, 1);
             // vmcnt(2*QN): tile 0 has landed, tile 1 may still be in flight
             static_assert(QN == 4 || QN == 8, "wait counts below are written for 4 or 8 loads per operand, wave and k-tile");
             if (QN == 8) __builtin_amdgcn_s_waitcnt(0x4F70);

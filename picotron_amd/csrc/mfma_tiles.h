@@ -78,43 +78,46 @@ constexpr int64_t kSplitWorkspaceBytes = (int64_t)kNumXcd * kCusPerXcd * BM * BN
 // `light_per_xcd` light ones (slots 0 .. per_xcd - 1).  With max_pieces > 1, the tiles left over after the full rounds of
 // kCusPerXcd (`rem` of them, slots >= full) are cut into `pieces` ranges of K each, so that the last, partly filled round
 // takes 1 / pieces of a tile instead of a whole one: slot full + t * pieces + p is piece p of tile slot full + t.
+// Tile and row totals fit 32 bits (the grid does), and everything here is 32-bit unsigned arithmetic on purpose: every
+// wavefront of every block runs this lookup on the CU's one scalar unit before its first load, and 64-bit divisions there
+// (some hundred scalar instructions each) were 2 % of a tile's time.
 struct GroupedLayout {
-    int64_t heavy, light, heavy_per_xcd, light_per_xcd, per_xcd;
-    int64_t full;  // slots of whole tiles that come first
+    uint32_t heavy, light, heavy_per_xcd, light_per_xcd, per_xcd;
+    uint32_t full;  // slots of whole tiles that come first
     int rem, pieces;
     int c0;        // this lane's counts[lane] (0 past E): the lookup that follows reuses it instead of loading it again
 };
 
 // Runs in every wave, 64 experts at a time (lane = expert): one coalesced load of counts[] per pass instead of a chain
-// of dependent scalar loads.  Tile and row totals fit 32 bits.
+// of dependent scalar loads.
 __device__ __forceinline__ GroupedLayout grouped_layout(const int64_t* counts, int E, int n_tiles, int max_pieces) {
     const int lane = threadIdx.x & 63;
     int heavy_m = 0, light_m = 0, c0 = 0;
     for (int base = 0; base < E; base += 64) {
-        const int c = base + lane < E ? (int)counts[base + lane] : 0, rem = c % BM;
-        if (base == 0) c0 = c;
-        heavy_m += c / BM + (rem > BM / 2);
+        const uint32_t c = base + lane < E ? (uint32_t)counts[base + lane] : 0u, rem = c % BM;
+        if (base == 0) c0 = (int)c;
+        heavy_m += (int)(c / BM) + (rem > BM / 2);
         light_m += (rem > 0 && rem <= BM / 2);
     }
     heavy_m = uniform_i32(wave_sum_i32(heavy_m));  // the same in every lane: scalar from here on
     light_m = uniform_i32(wave_sum_i32(light_m));
     GroupedLayout g;
     g.c0 = c0;
-    g.heavy = (int64_t)heavy_m * n_tiles;
-    g.light = (int64_t)light_m * n_tiles;
-    g.heavy_per_xcd = (g.heavy + kNumXcd - 1) / kNumXcd;
-    g.light_per_xcd = (g.light + kNumXcd - 1) / kNumXcd;
+    g.heavy = (uint32_t)heavy_m * (uint32_t)n_tiles;
+    g.light = (uint32_t)light_m * (uint32_t)n_tiles;
+    g.heavy_per_xcd = (g.heavy + kNumXcd - 1) / (uint32_t)kNumXcd;
+    g.light_per_xcd = (g.light + kNumXcd - 1) / (uint32_t)kNumXcd;
     g.per_xcd = g.heavy_per_xcd + g.light_per_xcd;
     g.full = g.per_xcd;
     g.rem = 0;
     g.pieces = 1;
     if (max_pieces > 1) {
-        const int rem = (int)(g.per_xcd % kCusPerXcd);
-        int pieces = rem == 0 ? 1 : kCusPerXcd / rem;
-        if (pieces > max_pieces) pieces = max_pieces;
-        if (pieces == 3) pieces = 2;
+        static_assert(kCusPerXcd == 32 && kMaxSplit == 4, "the piece count below is kCusPerXcd / rem, capped at 4, 3 -> 2");
+        const int rem = (int)(g.per_xcd % (uint32_t)kCusPerXcd);
+        int pieces = rem == 0 ? 1 : (rem <= 8 ? 4 : (rem <= 16 ? 2 : 1));
+        if (pieces > max_pieces) pieces = max_pieces == 3 ? 2 : max_pieces;
         if (pieces > 1) {
-            g.full = g.per_xcd - rem;
+            g.full = g.per_xcd - (uint32_t)rem;
             g.rem = rem;
             g.pieces = pieces;
         }
@@ -123,11 +126,11 @@ __device__ __forceinline__ GroupedLayout grouped_layout(const int64_t* counts, i
 }
 
 // Tile number `tile_slot` (0 .. per_xcd - 1) of XCD `xcd`.
-__device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, int n_tiles, const GroupedLayout& g, int64_t xcd,
-                                                 int64_t tile_slot, TileCoord* tc) {
+__device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, int n_tiles, const GroupedLayout& g, uint32_t xcd,
+                                                 uint32_t tile_slot, TileCoord* tc) {
     const int lane = threadIdx.x & 63;
     bool want_light;
-    int64_t L;
+    uint32_t L;
     if (tile_slot < g.heavy_per_xcd) {
         want_light = false;
         L = xcd * g.heavy_per_xcd + tile_slot;
@@ -139,52 +142,55 @@ __device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, i
     } else {
         return false;
     }
-    int64_t tiles_before = 0, rows_before = 0;
+    uint32_t tiles_before = 0, rows_before = 0;
     for (int base = 0; base < E; base += 64) {
-        const int c = base == 0 ? g.c0 : (base + lane < E ? (int)counts[base + lane] : 0), full = c / BM, rem = c % BM;
-        const int me = want_light ? (int)(rem > 0 && rem <= BM / 2) : full + (rem > BM / 2);
+        const uint32_t c = base == 0 ? (uint32_t)g.c0 : (base + lane < E ? (uint32_t)counts[base + lane] : 0u);
+        const uint32_t full = c / BM, rem = c % BM;
+        const int me = want_light ? (int)(rem > 0 && rem <= BM / 2) : (int)full + (rem > BM / 2);
         const int te = me * n_tiles;
-        const int te_incl = wave_scan_i32(te, lane), rows_incl = wave_scan_i32(c, lane);
-        const int te_total = uniform_i32(__shfl(te_incl, 63, 64));
+        const int te_incl = wave_scan_i32(te, lane), rows_incl = wave_scan_i32((int)c, lane);
+        const uint32_t te_total = (uint32_t)uniform_i32(__shfl(te_incl, 63, 64));
         if (L < tiles_before + te_total) {  // the tile belongs to an expert of this group of 64
-            const uint64_t hit = __ballot(tiles_before + te_incl > L);
+            const uint64_t hit = __ballot(tiles_before + (uint32_t)te_incl > L);
             const int src = uniform_i32(__ffsll((unsigned long long)hit) - 1);
-            const int c_e = __shfl(c, src, 64), me_e = __shfl(me, src, 64);
-            const int64_t Le = L - tiles_before - (__shfl(te_incl, src, 64) - __shfl(te, src, 64));
-            const int64_t start = rows_before + (__shfl(rows_incl, src, 64) - c_e);
-            const int m = want_light ? c_e / BM : (int)(Le % me_e);
-            // every lane holds the same numbers: hand them out as wave-uniform (scalar) values
-            tc->e = uniform_i32(base + src);
-            tc->m_tile = uniform_i32(m);
-            tc->n_tile = uniform_i32((int)(Le / me_e));
-            tc->row0 = uniform_i64(start + (int64_t)m * BM);
-            const int left = c_e - m * BM;
-            tc->rows = uniform_i32(left < BM ? left : BM);
+            const uint32_t c_e = (uint32_t)uniform_i32(__shfl((int)c, src, 64));
+            const uint32_t me_e = (uint32_t)uniform_i32(__shfl(me, src, 64));
+            const uint32_t Le = L - tiles_before - (uint32_t)uniform_i32(__shfl(te_incl, src, 64) - __shfl(te, src, 64));
+            const uint32_t start = rows_before + (uint32_t)uniform_i32(__shfl(rows_incl, src, 64)) - c_e;
+            const uint32_t nt = Le / me_e;
+            const uint32_t m = want_light ? c_e / BM : Le - nt * me_e;
+            tc->e = base + src;
+            tc->m_tile = (int)m;
+            tc->n_tile = (int)nt;
+            tc->row0 = (int64_t)(start + m * BM);
+            const uint32_t left = c_e - m * BM;
+            tc->rows = (int)(left < (uint32_t)BM ? left : (uint32_t)BM);
             tc->a_sn = n_tiles < 4 ? n_tiles : 4;
             tc->a_si = tc->n_tile % tc->a_sn;
-            tc->b_sn = uniform_i32(me_e < 8 ? me_e : 8);
-            tc->b_si = tc->m_tile % tc->b_sn;
+            tc->b_sn = (int)(me_e < 8 ? me_e : 8);
+            tc->b_si = (int)(m % (uint32_t)tc->b_sn);
             return true;
         }
         tiles_before += te_total;
-        rows_before += uniform_i32(__shfl(rows_incl, 63, 64));
+        rows_before += (uint32_t)uniform_i32(__shfl(rows_incl, 63, 64));
     }
     return false;
 }
 
 // The tile (and, with max_pieces > 1, the piece of it) behind position `slot` of this block's XCD's run (blockIdx.x / 8).
-__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, int64_t slot, TileCoord* tc,
+__device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, int n_tiles, uint32_t slot, TileCoord* tc,
                                                  int max_pieces = 1) {
     const GroupedLayout g = grouped_layout(counts, E, n_tiles, max_pieces);
-    int64_t tile_slot = slot;
+    uint32_t tile_slot = slot;
     tc->piece = 0;
     tc->pieces = 1;
     tc->ws_slot = 0;
     if (slot >= g.full && g.pieces > 1) {
-        const int64_t idx = slot - g.full;
-        if (idx >= (int64_t)g.rem * g.pieces) return false;
-        tile_slot = g.full + idx / g.pieces;
-        tc->piece = (int)(idx % g.pieces);
+        const uint32_t idx = slot - g.full;
+        if (idx >= (uint32_t)(g.rem * g.pieces)) return false;
+        const int lg = g.pieces >> 1;  // pieces is 2 or 4
+        tile_slot = g.full + (idx >> lg);
+        tc->piece = (int)(idx & (uint32_t)(g.pieces - 1));
         tc->pieces = g.pieces;
         tc->ws_slot = (int)((blockIdx.x % kNumXcd) * kCusPerXcd + idx);
     }
