@@ -121,7 +121,8 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     i32x8_t af[2][4], bfr[NJ];
     auto read_a = [&](int h, int i) { af[h][i] = read_frag(a_ad + (4 * h + i) * 2048); };
     auto read_b = [&](int j) { bfr[j] = read_frag(b_ad + j * 2048); };
-    // the 16 MFMAs (32 cycles each) of half h, B block by B block, with side(n) run after MFMA n: the slots for LDS
+    // the 16 MFMAs (32 cycles each) of half h, B block by B block (the B fragment first: the block comes out transposed,
+    // four neighbouring columns of a row per lane, as the epilogue stages them), with side(n) run after MFMA n: the slots for LDS
     // reads and loads.  After MFMA 4j + 3 nothing in this k-step needs bfr[j] any more.
     auto mma_with = [&](int h, auto active, auto side) {
 #pragma unroll
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if (decltype(active)::value)
-                    acc[4 * h + i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[h][i], bfr[j], acc[4 * h + i][j], 0, 0, 0, 0, 0, 0);
+                    acc[4 * h + i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bfr[j], af[h][i], acc[4 * h + i][j], 0, 0, 0, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 side(j * 4 + i);
                 __builtin_amdgcn_sched_barrier(0);
@@ -189,8 +190,10 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     __syncthreads();
 
     // epilogue: the two scales, rounding to bf16, and 32 rows at a time through a wave-private slice of LDS so that the
-    // stores are 16-byte lanes of contiguous rows.  A lane holds column (l & 15) and rows 4*(l >> 4) + r (r = 0..3) of
-    // each 16 x 16 accumulator block.
+    // stores are 16-byte lanes of contiguous rows.  The MFMAs take the B fragment as their first operand, so a lane holds
+    // row (l & 15) of each 16-row block and the four neighbouring columns 4*(l >> 4) .. +3 of each 16-column block: one
+    // row scale per block, four column scales per column block, two packed conversions and one 8-byte LDS write per
+    // four values.  (Widths are whole tiles here -- ffn_fp8_supported -- so only rows need bounds.)
     float* row_scale = (float*)(lds + kStageBytes);  // 256 floats, past the staging slices
     if (tid < BM) row_scale[tid] = p.x_scale[tc.row0 + (tid < tc.rows ? tid : tc.rows - 1)];
     constexpr int kEpiCols = MODE == kFp8GateUp ? CW / 2 : CW;
@@ -198,89 +201,127 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     char* epi = lds + wave * (32 * kEpiStride);
     constexpr int kChunksPerRow = kEpiCols / 8;
     constexpr int kReadIters = 32 * kChunksPerRow / 64;
-    auto stage_block = [&](auto value) {  // value(b, j, r): 16-row block b of the 32 rows, 16-column block j, row r of 4
+    constexpr int kRowsPerIt = 64 / kChunksPerRow;
+    const int c_row = lane / kChunksPerRow;        // the 16-byte chunk this lane reads back: row c_row + it * kRowsPerIt of the pass,
+    const int c_col = (lane % kChunksPerRow) * 8;  // columns c_col .. +7 of the wave's columns
+    auto lo16 = [](uint32_t v) { return __uint_as_float(v << 16); };
+    auto hi16 = [](uint32_t v) { return __uint_as_float(v & 0xFFFF0000u); };
+    auto pack4 = [](const f32x4_t& v) { return u32x2_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])}; };
+    auto stage_block = [&](auto packed) {  // packed(b, j): the four bf16 of 16-row block b of the 32 rows and 16-column block j
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int j = 0; j < kEpiCols / 16; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = b * 16 + g4 * 4 + r;
-                    *(uint16_t*)(epi + row * kEpiStride + (j * 16 + l15) * 2) = (uint16_t)f32_to_bf16_bits(value(b, j, r));
-                }
+                *(u32x2_t*)(epi + (b * 16 + l15) * kEpiStride + (j * 16 + 4 * g4) * 2) = packed(b, j);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    auto for_chunks = [&](int i, auto f) {
-#pragma unroll
-        for (int it = 0; it < kReadIters; ++it) {
-            const int idx = it * 64 + lane;
-            const int row = idx / kChunksPerRow, ch = idx % kChunksPerRow;
-            const u32x4_t v = *(const u32x4_t*)(epi + row * kEpiStride + ch * 16);
-            const int trow = wm * 128 + i * 32 + row;
-            if (trow < tc.rows) f(trow, ch * 8, v);
-        }
+    auto read_chunk = [&](int it) { return *(const u32x4_t*)(epi + (it * kRowsPerIt + c_row) * kEpiStride + c_col * 2); };
+    auto pass_live = [&](int i) { return wm * 128 + i * 32 < tc.rows; };  // wave-uniform
+    auto row_ok = [&](int i, int it) { return wm * 128 + i * 32 + it * kRowsPerIt + c_row < tc.rows; };
+    // f(std::true_type) when all 32 rows of pass i exist: that copy of the pass carries no bounds tests
+    auto with_fullness = [&](int i, auto f) {
+        if (wm * 128 + i * 32 + 32 <= tc.rows) f(std::true_type{});
+        else f(std::false_type{});
     };
     if (MODE == kFp8GateUp) {
         // g and u rounded to bf16 (what the two Linear outputs of the reference hold), then SwiGLU.  B blocks 0, 1 of the
         // wave are its 32 gate columns, blocks 2, 3 the up columns of the same FFN columns.
         const int64_t I = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * 128 + wn * (CW / 2);
-        float gs[2], us[2];
+        f32x4_t gs[2], us[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            gs[j] = p.g_scale[(int64_t)tc.e * I + col0 + j * 16 + l15];
-            us[j] = p.u_scale[(int64_t)tc.e * I + col0 + j * 16 + l15];
+            gs[j] = *(const f32x4_t*)(p.g_scale + (int64_t)tc.e * I + col0 + j * 16 + 4 * g4);
+            us[j] = *(const f32x4_t*)(p.u_scale + (int64_t)tc.e * I + col0 + j * 16 + 4 * g4);
         }
         __syncthreads();
+        const uint32_t off_act = (uint32_t)((c_row * (int)I + c_col) * 2);
+        const uint32_t off_gu = (uint32_t)((c_row * 2 * (int)I + c_col) * 2);
 #pragma unroll
         for (int i = 0; i < NI / 2; ++i) {
+            if (!pass_live(i)) continue;
+            u32x2_t gb[2][2], ub[2][2];
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < 2; ++b) {
+                const float sx = row_scale[wm * 128 + i * 32 + b * 16 + l15];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float sx = row_scale[wm * 128 + i * 32 + b * 16 + g4 * 4 + r];
+                for (int j = 0; j < 2; ++j) {
+                    f32x4_t g, u;
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        acc[2 * i + b][j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][j][r] * sx * gs[j]));
-                        acc[2 * i + b][2 + j][r] = bf16_bits_to_f32(f32_to_bf16_bits(acc[2 * i + b][2 + j][r] * sx * us[j]));
+                    for (int r = 0; r < 4; ++r) {
+                        g[r] = acc[2 * i + b][j][r] * sx * gs[j][r];
+                        u[r] = acc[2 * i + b][2 + j][r] * sx * us[j][r];
                     }
+                    gb[b][j] = pack4(g);
+                    ub[b][j] = pack4(u);
                 }
-            stage_block([&](int b, int j, int r) {
-                const float g = acc[2 * i + b][j][r], u = acc[2 * i + b][2 + j][r];
-                return bf16_bits_to_f32(f32_to_bf16_bits(g * sigmoid_fast(g))) * u;
-            });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.act + (tc.row0 + trow) * I + col0 + c) = v; });
-            if (p.inter13) {
-                stage_block([&](int b, int j, int r) { return acc[2 * i + b][j][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + col0 + c) = v; });
-                stage_block([&](int b, int j, int r) { return acc[2 * i + b][2 + j][r]; });
-                for_chunks(i, [&](int trow, int c, u32x4_t v) { *(u32x4_t*)(p.inter13 + (tc.row0 + trow) * 2 * I + I + col0 + c) = v; });
             }
+            stage_block([&](int b, int j) {
+                u32x2_t o;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float g0 = lo16(gb[b][j][h]), g1 = hi16(gb[b][j][h]);
+                    const uint32_t sl = pack_bf16x2(g0 * sigmoid_fast(g0), g1 * sigmoid_fast(g1));  // silu(g), rounded
+                    o[h] = pack_bf16x2(lo16(sl) * lo16(ub[b][j][h]), hi16(sl) * hi16(ub[b][j][h]));
+                }
+                return o;
+            });
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const int64_t r0 = tc.row0 + wm * 128 + i * 32;
+                char* act_base = (char*)(p.act + r0 * I + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it)
+                    if (kFull || row_ok(i, it)) *(u32x4_t*)(act_base + (int64_t)it * kRowsPerIt * I * 2 + off_act) = read_chunk(it);
+                if (p.inter13) {
+                    char* gu_base = (char*)(p.inter13 + r0 * 2 * I + col0);
+                    stage_block([&](int b, int j) { return gb[b][j]; });
+#pragma unroll
+                    for (int it = 0; it < kReadIters; ++it)
+                        if (kFull || row_ok(i, it)) *(u32x4_t*)(gu_base + (int64_t)it * kRowsPerIt * I * 4 + off_gu) = read_chunk(it);
+                    stage_block([&](int b, int j) { return ub[b][j]; });
+#pragma unroll
+                    for (int it = 0; it < kReadIters; ++it)
+                        if (kFull || row_ok(i, it))
+                            *(u32x4_t*)(gu_base + I * 2 + (int64_t)it * kRowsPerIt * I * 4 + off_gu) = read_chunk(it);
+                }
+            });
         }
     } else {
         // y = bf16(acc * row scale * column scale), times the row weight (rounded again) when there is one
         const int64_t H = p.N;
         const int64_t col0 = (int64_t)tc.n_tile * BN + wn * CW;
-        float ws[NJ];
+        f32x4_t ws[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) ws[j] = p.g_scale[(int64_t)tc.e * H + col0 + j * 16 + l15];
+        for (int j = 0; j < NJ; ++j) ws[j] = *(const f32x4_t*)(p.g_scale + (int64_t)tc.e * H + col0 + j * 16 + 4 * g4);
         __syncthreads();
+        const uint32_t off = (uint32_t)((c_row * (int)H + c_col) * 2);
 #pragma unroll
         for (int i = 0; i < NI / 2; ++i) {
-            if (wm * 128 + i * 32 >= tc.rows) continue;  // wave-uniform
-            stage_block([&](int b, int j, int r) {
-                return acc[2 * i + b][j][r] * row_scale[wm * 128 + i * 32 + b * 16 + g4 * 4 + r] * ws[j];
-            });
-            for_chunks(i, [&](int trow, int c, u32x4_t v) {
-                const int64_t grow = tc.row0 + trow;
-                if (p.row_weight) {
-                    const float rw = bf16_bits_to_f32(p.row_weight[grow]);
+            if (!pass_live(i)) continue;
+            stage_block([&](int b, int j) {
+                const float sx = row_scale[wm * 128 + i * 32 + b * 16 + l15];
+                f32x4_t v;
 #pragma unroll
-                    for (int w2 = 0; w2 < 4; ++w2)
-                        v[w2] = pack_bf16x2(__uint_as_float(v[w2] << 16) * rw, __uint_as_float(v[w2] & 0xFFFF0000u) * rw);
+                for (int r = 0; r < 4; ++r) v[r] = acc[2 * i + b][j][r] * sx * ws[j][r];
+                return pack4(v);
+            });
+            with_fullness(i, [&](auto full) {
+                constexpr bool kFull = decltype(full)::value;
+                const int64_t r0 = tc.row0 + wm * 128 + i * 32;
+                char* out_base = (char*)(p.act + r0 * H + col0);
+#pragma unroll
+                for (int it = 0; it < kReadIters; ++it) {
+                    if (!(kFull || row_ok(i, it))) continue;
+                    u32x4_t v = read_chunk(it);
+                    if (p.row_weight) {
+                        const float rw = bf16_bits_to_f32(p.row_weight[r0 + it * kRowsPerIt + c_row]);
+#pragma unroll
+                        for (int w2 = 0; w2 < 4; ++w2) v[w2] = pack_bf16x2(lo16(v[w2]) * rw, hi16(v[w2]) * rw);
+                    }
+                    *(u32x4_t*)(out_base + (int64_t)it * kRowsPerIt * H * 2 + off) = v;
                 }
-                *(u32x4_t*)(p.act + grow * H + col0 + c) = v;
             });
         }
     }
