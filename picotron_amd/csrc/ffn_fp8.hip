@@ -19,6 +19,7 @@ namespace {
 
 constexpr int kFp8Waves = 8;
 constexpr int kFp8BK = 128;  // k values (bytes) per k-step
+constexpr int kFp8PrefetchDist = 2;
 
 typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 
@@ -87,6 +88,38 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         }
     };
 
+    // L2 prefetch, as in the bf16 kernels: every k-step each wave touches (one 4-byte load per 128-byte line into a register
+    // nobody reads) its share of the lines of an operand slice kFp8PrefetchDist k-steps ahead -- the first half of the waves lines
+    // of the A slice, the second half lines of the B slice -- so that the demand loads of the tiles that share the slice do not
+    // queue behind the same misses.
+    const char* pf_cur;
+    {
+        const bool pf_b = wave >= kFp8Waves / 2;
+        const int q = (wave % (kFp8Waves / 2)) * 64 + lane;
+        const int si = pf_b ? tc.b_si : tc.a_si, sn = pf_b ? tc.b_sn : tc.a_sn;
+        int j = sn > 1 ? si + sn * q : q;  // line of the 256-line slice (one line per row)
+        if (j >= 256) j = si;
+        if (!pf_b) {
+            const int r = j < tc.rows ? j : tc.rows - 1;
+            pf_cur = (const char*)(p.xq + (tc.row0 + r) * p.K);
+        } else if (MODE == kFp8GateUp) {
+            const uint8_t* m = j < 128 ? p.gq : p.uq;
+            pf_cur = (const char*)(m + ((int64_t)tc.e * p.N + (int64_t)tc.n_tile * 128 + (j & 127)) * p.K);
+        } else {
+            pf_cur = (const char*)(p.gq + ((int64_t)tc.e * p.N + (int64_t)tc.n_tile * BN + j) * p.K);
+        }
+        const int kt0 = kFp8PrefetchDist < n_kt ? kFp8PrefetchDist : (n_kt > 0 ? n_kt - 1 : 0);
+        pf_cur += (int64_t)kt0 * kFp8BK;
+    }
+    // the touch in front of the loop takes k-tile kFp8PrefetchDist, the one of k-step kt k-tile kt + kFp8PrefetchDist + 1 (its operand
+    // loads go out a k-step later); past the last k-tile the pointer stays where it is
+    int pf_kt = kFp8PrefetchDist;
+    auto prefetch_l2 = [&]() {
+        asm volatile("global_load_dword v255, %0, off" ::"v"(pf_cur) : "v255", "memory");
+        ++pf_kt;
+        if (pf_kt < n_kt) pf_cur += kFp8BK;
+    };
+
     // LDS -> fragments.  An MFMA takes all 128 k values of a row: lane (row l & 15 of a 16-row block, k group l >> 4)
     // supplies the 32 bytes of k group l >> 4, the 16-byte chunks 2*(l >> 4) and 2*(l >> 4) + 1 of its row; with the XOR
     // swizzle the second is the address of the first XOR 16.  The swizzle depends on (row >> 1) & 7 only, which is the
@@ -141,7 +174,8 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         issue_tile(0, 0);
         if (n_kt > 1) {
             issue_tile(1, 1);
-            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): tile 0 has landed, tile 1 may still be in flight
+            prefetch_l2();  // from here on the youngest load in flight is always a prefetch touch
+            __builtin_amdgcn_s_waitcnt(0x0F79);  // vmcnt(9): tile 0 has landed, tile 1 and the touch may still be in flight
         } else {
             __builtin_amdgcn_s_waitcnt(0x0F70);
         }
@@ -167,7 +201,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
             mma_with(0, active, [&](int n) {
                 if (kActive && (n & 1) == 0 && n < 8) read_a(1, n >> 1);
             });
-            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __builtin_amdgcn_s_waitcnt(0x0F71);  // the operand loads of a k-step ago have landed; the prefetch touch issued after them may stay in flight
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_barrier();
@@ -181,6 +215,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
                 // past the last tile these read a stage that is not used any more
                 if (kActive && (n & 3) == 3) read_b(n >> 2);
                 if (kActive && n >= 8 && n < 12) read_a(0, n - 8);
+                if (n == 13) prefetch_l2();
             });
         }
     };
