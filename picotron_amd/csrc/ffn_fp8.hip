@@ -88,6 +88,12 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
         }
     };
 
+    // the first two k-tiles go out before the rest of the set-up (prefetch pointer, fragment addresses, zeroed accumulators)
+    if (n_kt > 0) {
+        issue_tile(0, 0);
+        if (n_kt > 1) issue_tile(1, 1);
+    }
+
     // L2 prefetch, as in the bf16 kernels: every k-step each wave touches (one 4-byte load per 128-byte line into a register
     // nobody reads) its share of the lines of an operand slice kFp8PrefetchDist k-steps ahead -- the first half of the waves lines
     // of the A slice, the second half lines of the B slice -- so that the demand loads of the tiles that share the slice do not
@@ -171,9 +177,7 @@ __global__ __launch_bounds__(kFp8Waves * 64, 1) void ffn_fp8_kernel(Fp8Params p)
     };
 
     if (n_kt > 0) {
-        issue_tile(0, 0);
         if (n_kt > 1) {
-            issue_tile(1, 1);
             prefetch_l2();  // from here on the youngest load in flight is always a prefetch touch
             __builtin_amdgcn_s_waitcnt(0x0F79);  // vmcnt(9): tile 0 has landed, tile 1 and the touch may still be in flight
         } else {
