@@ -184,7 +184,7 @@ class GemmTimer:
                 en.record()
                 label = name
                 if name == "wgrad":  # (lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset)
-                    label = "wgrad_down" if a[1] == a[7] else ("wgrad_up" if kw.get("lhs_offset", 0) else "wgrad_gate")
+                    label = "wgrad_" + kw["which"]  # down, gate, up, or gate_up: both in one launch
                     n_experts, rows = a[5], a[6]
                 else:  # (x, counts, weight, ...): weight [E, ., .]
                     n_experts, rows = a[2].shape[0], a[0].shape[0]
@@ -203,7 +203,8 @@ class GemmTimer:
             # routed launches: the rows that reach the GEMMs (kept rows under a capacity limit); shared: all tokens
             n_rows = rows if label.startswith("shared_") else routed_rows
             i_dim = I * self.shared_mult if label.startswith("shared_") else I
-            d = per.setdefault(label, {"ms": 0.0, "n": 0, "flop": self.FLOP[name] * n_rows * H * i_dim})
+            flop_per = self.FLOP[name] * (2.0 if label.endswith("wgrad_gate_up") else 1.0)
+            d = per.setdefault(label, {"ms": 0.0, "n": 0, "flop": flop_per * n_rows * H * i_dim})
             d["ms"] += st.elapsed_time(en)
             d["n"] += 1
         return {k: (v["ms"] / v["n"], v["flop"], v["n"]) for k, v in per.items()}

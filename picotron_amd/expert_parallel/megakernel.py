@@ -216,7 +216,9 @@ def _dgrad_x(d13, counts, gate_w, up_w):
     return dx
 
 
-def _wgrad(lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset=0):
+def _wgrad(lhs, ld_lhs, rhs, ld_rhs, counts, E, N, P, Q, dtype, device, lhs_offset=0, which=None):
+    """out [E, P, Q] = per expert lhs_e^T @ rhs_e.  ``which`` ("down", "gate", "up", "gate_up") names the weight gradient for
+    timing hooks; it does not change the call."""
     lib = _lib.load()
     out = torch.empty((E, P, Q), dtype=dtype, device=device)
     lhs_ptr = _lib.ctypes.c_void_p(lhs.data_ptr() + lhs_offset * lhs.element_size())
@@ -261,9 +263,9 @@ def fused_moe_wgrad(x_sorted, counts, a, d_inter13, dy):
     x, a, d13, dy = x_sorted.contiguous(), a.contiguous(), d_inter13.contiguous(), dy.contiguous()
     counts = _counts64(counts, x.device)
     E, N, H, I = counts.numel(), x.shape[0], x.shape[1], a.shape[1]
-    d_down = _wgrad(dy, H, a, I, counts, E, N, H, I, x.dtype, x.device)
-    d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
-    d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
+    d_down = _wgrad(dy, H, a, I, counts, E, N, H, I, x.dtype, x.device, which="down")
+    d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, which="gate")
+    d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I, which="up")
     return d_gate, d_up, d_down
 
 
@@ -327,11 +329,16 @@ class _FusedMoE(torch.autograd.Function):
             if want_dx:
                 dx = _dgrad_x(d13, counts, gw, uw)
         if want_down:
-            d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device)
-        if want_gate:
-            d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device)
-        if want_up:
-            d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I)
+            d_down = _wgrad(dy, H, act, I, counts, E, N, H, I, x.dtype, x.device, which="down")
+        if want_gate and want_up:
+            # one launch for both: [dg | du] is the left operand as it lies (2I columns), the result [E, 2I, H] holds
+            # d gate_w[e] and d up_w[e] one after the other, and each expert's slice of either is contiguous
+            d_gu = _wgrad(d13, 2 * I, x, H, counts, E, N, 2 * I, H, x.dtype, x.device, which="gate_up")
+            d_gate, d_up = d_gu[:, :I], d_gu[:, I:]
+        elif want_gate:
+            d_gate = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, which="gate")
+        elif want_up:
+            d_up = _wgrad(d13, 2 * I, x, H, counts, E, N, I, H, x.dtype, x.device, lhs_offset=I, which="up")
         return dx, d_gate, d_up, d_down, None, d_rw, None
 
 
