@@ -5,7 +5,9 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is only enqueued,
  *     nothing synchronises, allocates or keeps a pointer past the call;
  *   - returns 0 on success, PICOMOE_ERR_ARG for a shape / dtype / alignment the kernels do not
- *     accept, or PICOMOE_ERR_HIP_BASE + hipError_t when the launch itself failed;
+ *     accept, PICOMOE_ERR_TOO_LARGE for one whose tile count does not fit the kernels' 32-bit tile numbering
+ *     (expert FFN: about (n_rows / 64 + experts) x max(hidden, 2 inter) / 64 >= 2^31), or PICOMOE_ERR_HIP_BASE +
+ *     hipError_t when the launch itself failed;
  *   - `dtype` is PICOMOE_F32 or PICOMOE_BF16 (the dtype of the token features / weights).
  *
  * Each declaration cites the reference code it replaces (paths inside the picotron checkout,

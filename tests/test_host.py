@@ -49,6 +49,11 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.picomoe_ffn_dgrad_x(null, counts, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 0
     assert lib.picomoe_ffn_down(null, counts, 4, 8, 256, 128, null, null, 1, null, null, 0, null) == 1    # null tensors
     assert lib.picomoe_ffn_down(null, null, 4, 0, 256, 128, null, null, 1, null, null, 0, null) == 1      # null counts
+    # shapes whose tiles cannot be numbered in 32 bits are refused (PICOMOE_ERR_TOO_LARGE = 2) before anything is touched
+    big_rows, big_width = 2**31 - 1, 2**24
+    assert lib.picomoe_ffn_gate_up(null, counts, 4, big_rows, 256, big_width, null, null, 1, null, null, null, 0, null) == 2
+    assert lib.picomoe_ffn_dgrad_x(null, counts, 4, big_rows, big_width, 256, null, null, 1, null, null, 0, null) == 2
+    assert lib.picomoe_ffn_wgrad(counts, 2**26, counts, 2**26, counts, 1024, 8, 2**26, 2**26, 1, counts, null) == 2
     # diagnostics and queries
     assert lib.picomoe_diag_mfma_loop_flop(0, 10, 2) == 64 * 2 * 16 * 16 * 32 * 8 * 10 * 2
     assert lib.picomoe_diag_mfma_loop_flop(9, 10, 2) == -1
