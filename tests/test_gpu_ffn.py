@@ -102,6 +102,28 @@ def test_empty_input_and_all_empty_but_one(gpu):
     assert torch.allclose(y.cpu(), O.expert_ffn(x, counts, gw, uw, dw), atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype,H,I", [(torch.float32, 40, 72), (torch.bfloat16, 256, 384), (torch.bfloat16, 320, 192)])
+def test_gate_and_up_weight_gradients_in_one_launch(gpu, dtype, H, I):
+    """The autograd path computes d gate_w and d up_w with one launch ([dg | du] as the left operand in place, the result
+    [E, 2I, H] split into two views); fused_moe_wgrad keeps one launch each.  Same tiles, same arithmetic: bit-equal, and
+    every expert's slice of either gradient is contiguous (what the per-expert parameters receive)."""
+    from picotron_amd.expert_parallel import megakernel
+
+    E = 4
+    x, counts, gw, uw, dw, g = _mk(E, H, I, [300, 0, 5, 257], dtype, 11)
+    dy = torch.randn(x.shape, generator=g).to(dtype)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, gw, uw, dw)]
+    megakernel.fused_moe(leaves[0], counts.cuda(), *leaves[1:]).backward(dy.cuda())
+    _, a, d13 = megakernel.fused_moe_dgrad(x.cuda(), counts.cuda(), gw.cuda(), uw.cuda(), dw.cuda(), dy.cuda())
+    dg, du, dd = megakernel.fused_moe_wgrad(x.cuda(), counts.cuda(), a, d13, dy.cuda())
+    assert torch.equal(leaves[1].grad, dg) and torch.equal(leaves[2].grad, du) and torch.equal(leaves[3].grad, dd)
+    # only one of the two asked for: the separate launches
+    only_up = [t.cuda() for t in (x, gw, uw, dw)]
+    only_up[2].requires_grad_(True)
+    megakernel.fused_moe(only_up[0], counts.cuda(), *only_up[1:]).backward(dy.cuda())
+    assert torch.equal(only_up[2].grad, du) and only_up[1].grad is None
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_explicit_dgrad_wgrad_api(gpu, dtype):
     """fused_moe_dgrad / fused_moe_wgrad return the intermediates the reference documents (a, d_inter13)."""
