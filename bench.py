@@ -40,7 +40,7 @@ MEASURED_TRAFFIC = {
     "c5": {"bytes": 35.3e9, "algorithmic_bytes": 15.5e9, "sources": "d6e1eef8dff7e27b",
            "files": ("ffn_mfma.hip", "mfma_tiles.h", "ffn.h", "common.h"),
            "summary": "profiles/ffn_mfma_kernel_mixtral_hbm_traffic.txt"},
-    "c2": {"bytes": 201.6e6, "algorithmic_bytes": 201.4e6, "sources": "8ac0240fe279f58b",
+    "c2": {"bytes": 201.6e6, "algorithmic_bytes": 201.4e6, "sources": "567861dc6e2a9e36",
            "files": ("fp8_quant.hip", "common.h"),
            "summary": "profiles/quant_bf16_wave_per_row_fp8_round_trip.txt"},
 }

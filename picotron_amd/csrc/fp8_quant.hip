@@ -536,8 +536,8 @@ extern "C" const char* picomoe_error_string(int code) {
     if (code == PICOMOE_OK) return "ok";
     if (code == PICOMOE_ERR_ARG) return "picomoe: unsupported shape, dtype, alignment or null pointer";
     if (code == PICOMOE_ERR_TOO_LARGE)
-        return "picomoe: the input is larger than the fixed scratch of this no-allocation entry point "
-               "(use the variant that takes a workspace)";
+        return "picomoe: too large -- the input exceeds the fixed scratch of a no-allocation entry point (use the variant that "
+               "takes a workspace), or an expert-FFN shape has more tiles than the kernels' 32-bit tile numbering holds";
     if (code >= PICOMOE_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(code - PICOMOE_ERR_HIP_BASE));
     return "picomoe: unknown error code";
 }
