@@ -30,7 +30,7 @@ extern "C" {
 #define PICOMOE_F32 0
 #define PICOMOE_BF16 1
 
-#define PICOMOE_ABI_VERSION 5
+#define PICOMOE_ABI_VERSION 6
 
 /* ABI version of the loaded library (compare with PICOMOE_ABI_VERSION). */
 int picomoe_abi_version(void);
@@ -88,6 +88,22 @@ int picomoe_route_bwd(const float* probs, const int64_t* topk_idx, const void* d
  * (skipped when expert_bias is NULL or bias_rate == 0). */
 int picomoe_balance(const int* counts, const float* colsum_partial, int n_partials, int64_t n_tokens, int num_experts,
                     int top_k, float aux_coef, float bias_rate, float* aux_out, float* expert_bias, void* stream);
+
+/* Backward of the router's gate Linear, EP/expert_parallel.py:65 and :174 (`self.gate = nn.Linear(hidden, num_experts,
+ * bias=False)`, `router_logits = self.gate(tokens)`: autograd's d_tokens = d_logits @ gate.weight and d_weight =
+ * d_logits.T @ tokens), together with autograd's sum of the tokens' gradient paths (through the router and through the
+ * experts), in one pass over the tokens: d_x[t] = addend[t] + d_logits[t] @ gate_w and, when d_w is given,
+ * d_w[e] = sum_t d_logits[t, e] * tokens[t] (fp32 sums in a fixed order, rounded once).  d_logits [n_tokens, num_experts],
+ * gate_w and d_w [num_experts, hidden], addend (NULL = zeros), tokens and d_x [n_tokens, hidden], all in dtype; the product
+ * d_logits @ gate_w is rounded to dtype before the sum with the addend, as a GEMM followed by an add rounds.
+ * num_experts <= 16 for d_x alone (tokens, d_w, workspace NULL) and <= 8 with d_w, which needs `workspace` of
+ * picomoe_gate_bwd_workspace_bytes(...) bytes (0 = this gate has no fused weight gradient; -1 = bad arguments); hidden a
+ * multiple of 16 bytes, pointers 16-byte aligned: PICOMOE_ERR_ARG otherwise (a caller keeps the library GEMMs for wider
+ * routers). */
+int64_t picomoe_gate_bwd_workspace_bytes(int dtype, int64_t n_tokens, int num_experts, int64_t hidden);
+int picomoe_gate_bwd(const void* d_logits, const void* gate_w, const void* addend, const void* tokens, int dtype,
+                     int64_t n_tokens, int num_experts, int64_t hidden, void* d_x, void* d_w, void* workspace,
+                     int64_t workspace_bytes, void* stream);
 
 /* ---- Permute / unpermute (the EP=1 form of dispatch / combine) ---------------------------------------
  * Replaces EP/expert_parallel.py:30-35 and :335-339 (stable argsort by expert, its inverse, bincount) and

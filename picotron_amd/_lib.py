@@ -12,7 +12,7 @@ import torch
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libpicomoe.so")
 HEADER_PATH = os.path.join(os.path.dirname(_PKG_DIR), "include", "picomoe.h")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -30,6 +30,8 @@ _SIGNATURES = {
     "picomoe_route_fwd": [_p, _i32, _i64, _i32, _i32, _p, _i32, _p, _p, _p, _p, _p, _p],
     "picomoe_route_bwd": [_p, _p, _p, _i32, _i64, _i32, _i32, _i32, _p, _p, _f32, _p, _p],
     "picomoe_balance": [_p, _p, _i32, _i64, _i32, _i32, _f32, _f32, _p, _p, _p],
+    "picomoe_gate_bwd_workspace_bytes": [_i32, _i64, _i32, _i64],
+    "picomoe_gate_bwd": [_p, _p, _p, _p, _i32, _i64, _i32, _i64, _p, _p, _p, _i64, _p],
     "picomoe_permute_workspace_bytes": [_i64, _i32],
     "picomoe_permute_plan": [_p, _i64, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
     "picomoe_permute_plan_static_max_bytes": [],
@@ -52,7 +54,7 @@ _SIGNATURES = {
 }
 _RESTYPES = {"picomoe_error_string": ctypes.c_char_p, "picomoe_permute_workspace_bytes": ctypes.c_int64,
              "picomoe_permute_plan_static_max_bytes": ctypes.c_int64,
-             "picomoe_ffn_workspace_bytes": ctypes.c_int64, "picomoe_diag_mfma_loop_flop": ctypes.c_int64}
+             "picomoe_ffn_workspace_bytes": ctypes.c_int64, "picomoe_gate_bwd_workspace_bytes": ctypes.c_int64, "picomoe_diag_mfma_loop_flop": ctypes.c_int64}
 
 _lib = None
 

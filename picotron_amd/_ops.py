@@ -83,6 +83,76 @@ class _Route(torch.autograd.Function):
         return d_logits, None, None, None, None, None, None
 
 
+GATE_DGRAD_MAX_EXPERTS = 16
+
+
+def gate_dgrad_supported(tokens, weight):
+    """Whether picomoe_gate_bwd takes this gate: up to 16 experts, fp32 or bf16 in one dtype, rows of whole 16-byte chunks."""
+    return (tokens.is_cuda and tokens.dim() == 2 and weight.dim() == 2 and tokens.dtype == weight.dtype
+            and tokens.dtype in (torch.float32, torch.bfloat16) and weight.shape[0] <= GATE_DGRAD_MAX_EXPERTS
+            and (tokens.shape[1] * tokens.element_size()) % 16 == 0 and not torch.is_autocast_enabled())
+
+
+def gate_bwd(d_logits, weight, addend, tokens, want_weight_grad):
+    """(d_tokens, d_weight or None) of ``linear(tokens, weight)`` with ``addend`` (the tokens' gradient from their other
+    readers, or None) summed in: one pass over the tokens.  d_weight is None when it was not asked for or the kernel has no
+    fused form for this many experts (the caller then runs the GEMM)."""
+    lib = _lib.load()
+    T, H = tokens.shape
+    E = weight.shape[0]
+    dt = _lib.dtype_code(tokens.dtype)
+    d_logits, weight, tokens = d_logits.contiguous(), weight.contiguous(), tokens.contiguous()
+    addend = addend.to(tokens.dtype).contiguous() if addend is not None else None
+    d_tokens = _empty((T, H), tokens.dtype, tokens.device)
+    ws_bytes = lib.picomoe_gate_bwd_workspace_bytes(dt, T, E, H) if want_weight_grad else 0
+    if ws_bytes < 0:
+        raise _lib.PicomoeError(f"picomoe_gate_bwd_workspace_bytes refused {T} tokens x {E} experts x {H}")
+    d_weight = ws = None
+    if ws_bytes > 0:
+        d_weight = _empty((E, H), tokens.dtype, tokens.device)
+        ws = _empty((ws_bytes,), torch.uint8, tokens.device)
+    _lib.check(
+        lib.picomoe_gate_bwd(_lib.ptr(d_logits), _lib.ptr(weight), _lib.ptr(addend), _lib.ptr(tokens) if d_weight is not None else None,
+                             dt, T, E, H, _lib.ptr(d_tokens), _lib.ptr(d_weight), _lib.ptr(ws), ws_bytes, _lib.stream_ptr()),
+        "picomoe_gate_bwd",
+    )
+    return d_tokens, d_weight
+
+
+class _GateTap(torch.autograd.Function):
+    """(logits, tokens) = (tokens @ weight.T, tokens): the router's gate Linear with the tokens handed through.
+
+    Everything else that reads the tokens (dispatch, shared expert) reads the second output, so autograd delivers the sum
+    of their gradients here together with d_logits, and one kernel writes d_tokens = that sum + d_logits @ weight and, for
+    up to 8 experts, d_weight = d_logits.T @ tokens -- where an ``nn.Linear`` node beside the others costs a GEMM that
+    writes [T, H], an add that reads two and writes one, and a GEMM with an E-row output that reads the tokens at a
+    fraction of the memory rate.  The logits stay a library GEMM, as in the reference (expert_parallel.py:65, :174).
+    """
+
+    @staticmethod
+    def forward(ctx, tokens, weight):
+        ctx.save_for_backward(tokens, weight)
+        ctx.set_materialize_grads(False)
+        return torch.nn.functional.linear(tokens, weight), tokens
+
+    @staticmethod
+    def backward(ctx, d_logits, d_tap):
+        tokens, weight = ctx.saved_tensors
+        if d_logits is None:
+            return (d_tap if ctx.needs_input_grad[0] else None), None
+        d_tokens = d_weight = None
+        if ctx.needs_input_grad[0]:
+            d_tokens, d_weight = gate_bwd(d_logits, weight, d_tap, tokens, ctx.needs_input_grad[1])
+        if ctx.needs_input_grad[1] and d_weight is None:
+            d_weight = d_logits.t() @ tokens
+        return d_tokens, d_weight
+
+
+def gate_tap(tokens, weight):
+    """Router logits and the tokens to hand to every other reader of them (see _GateTap); needs gate_dgrad_supported."""
+    return _GateTap.apply(tokens, weight)
+
+
 def route(logits, bias_f32, top_k, norm_topk, balance=False, aux_coef=0.0, bias_rate=0.0):
     """Returns (topk_idx int64 [T,k], topk_w [T,k] in logits.dtype, aux fp32 scalar)."""
     return _Route.apply(logits, bias_f32, top_k, norm_topk, balance, aux_coef, bias_rate)

@@ -341,6 +341,244 @@ void launch_route_bwd(const RouteShape& rs, unsigned blocks, hipStream_t st, con
     });
 }
 
+// ---- gradient of the gate Linear towards the tokens ---------------------------------------------------------------
+// d_x[t, :] = addend[t, :] + d_logits[t, :] @ W,  W [E, hidden] with E <= 16: an [n_tokens, E] x [E, hidden] product is E
+// multiply-adds per element written, so the pass is paid in bytes; done beside the sum of the tokens' two gradient paths
+// (router and experts) it costs one read and one write of [n_tokens, hidden] where a GEMM followed by an add costs a
+// write, two reads and a write.  A thread keeps its V columns of all E rows of W in registers and walks the tokens of its
+// block; the E gradient logits of a token are loaded by the first E lanes and handed round as scalars.
+// Rounding: the product is rounded to T, then the sum with the addend is rounded to T (a GEMM in T followed by an add in T).
+template <typename T, int V>
+struct Cols;
+template <>
+struct Cols<uint16_t, 8> {
+    typedef u32x4_t raw_t;
+    static __device__ __forceinline__ void widen(raw_t r, float (&f)[8]) {
+        const uint32_t a[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(a[i] << 16);
+            f[2 * i + 1] = __uint_as_float(a[i] & 0xFFFF0000u);
+        }
+    }
+    static __device__ __forceinline__ raw_t narrow(const float (&f)[8]) {
+        return raw_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+    }
+    // every value rounded to bf16 and widened again: the packed conversion, then the two halves of each word
+    static __device__ __forceinline__ void round_all(float (&f)[8]) { widen(narrow(f), f); }
+};
+template <>
+struct Cols<float, 4> {
+    typedef f32x4_t raw_t;
+    static __device__ __forceinline__ void widen(raw_t r, float (&f)[4]) { f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w; }
+    static __device__ __forceinline__ raw_t narrow(const float (&f)[4]) { return raw_t{f[0], f[1], f[2], f[3]}; }
+    static __device__ __forceinline__ void round_all(float (&)[4]) {}
+};
+
+constexpr int kGateDgradMaxExperts = 16;
+constexpr int kGateDgradTokensInFlight = 4;
+
+template <typename T, int V, int EMAX>
+__global__ __launch_bounds__(256) void gate_dgrad_kernel(const T* __restrict__ d_logits, const T* __restrict__ w,
+                                                         const T* __restrict__ addend, int64_t n_tokens, int E, int64_t hidden,
+                                                         T* __restrict__ out) {
+    typedef Cols<T, V> C;
+    typedef typename C::raw_t raw_t;
+    const int lane = threadIdx.x & 63;
+    const int64_t col = ((int64_t)blockIdx.y * 256 + threadIdx.x) * V;
+    const bool live = col < hidden;  // hidden is a multiple of V: a thread's columns are all inside or all outside
+    float wr[EMAX][V];
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) wr[e][i] = 0.f;
+        if (e < E && live) C::widen(*(const raw_t*)(w + (int64_t)e * hidden + col), wr[e]);
+    }
+    constexpr int U = kGateDgradTokensInFlight;
+    for (int64_t t0 = blockIdx.x; t0 < n_tokens; t0 += (int64_t)gridDim.x * U) {
+        raw_t a[U];
+        float dl[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t t = t0 + (int64_t)u * gridDim.x;
+            dl[u] = 0.f;
+            if (t < n_tokens) {  // uniform over the block
+                if (lane < E) dl[u] = to_f32<T>(d_logits[t * E + lane]);
+                if (addend && live) a[u] = *(const raw_t*)(addend + t * hidden + col);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t t = t0 + (int64_t)u * gridDim.x;
+            if (t >= n_tokens) break;
+            float acc[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = 0.f;
+#pragma unroll
+            for (int e = 0; e < EMAX; ++e) {
+                const float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(dl[u]), e));  // 0 for e >= E
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] = fmaf(d, wr[e][i], acc[i]);
+            }
+            if (addend) {
+                float av[V];
+                if (live) C::widen(a[u], av);
+                C::round_all(acc);
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] += live ? av[i] : 0.f;
+            }
+            if (live) *(raw_t*)(out + t * hidden + col) = C::narrow(acc);
+        }
+    }
+}
+
+template <typename T, int V>
+void launch_gate_dgrad(hipStream_t st, const void* d_logits, const void* w, const void* addend, int64_t n_tokens, int E,
+                       int64_t hidden, void* out) {
+    const int64_t cols_per_block = 256 * V;
+    const dim3 grid((unsigned)(n_tokens < 512 ? n_tokens : 512), (unsigned)((hidden + cols_per_block - 1) / cols_per_block));
+    if (E <= 8)
+        gate_dgrad_kernel<T, V, 8><<<grid, dim3(256), 0, st>>>((const T*)d_logits, (const T*)w, (const T*)addend, n_tokens, E,
+                                                               hidden, (T*)out);
+    else
+        gate_dgrad_kernel<T, V, kGateDgradMaxExperts><<<grid, dim3(256), 0, st>>>((const T*)d_logits, (const T*)w,
+                                                                                  (const T*)addend, n_tokens, E, hidden, (T*)out);
+}
+
+// The same pass with the gate's weight gradient beside it: d_w[e, :] = sum_t d_logits[t, e] * x[t, :] is E more
+// multiply-adds per element of x read, against columns the thread already owns, so reading x here (one more stream)
+// replaces a GEMM with an 8-row output that runs at a fifth of the memory rate.  A block's four wavefronts own the same
+// 64 * V columns and every fourth token of the block's share; their sums meet in LDS in wave order, the blocks' sums in
+// `partial` [gridDim.x][E][hidden] fp32, which gate_wgrad_reduce_kernel adds in block order: no atomics, one fixed order.
+constexpr int kGateBwdMaxExperts = 8;
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void gate_bwd_kernel(const T* __restrict__ d_logits, const T* __restrict__ w,
+                                                       const T* __restrict__ addend, const T* __restrict__ x, int64_t n_tokens,
+                                                       int E, int64_t hidden, T* __restrict__ d_x, float* __restrict__ partial) {
+    typedef Cols<T, V> C;
+    typedef typename C::raw_t raw_t;
+    constexpr int EMAX = kGateBwdMaxExperts;
+    __shared__ float red[3][EMAX * V][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t col = ((int64_t)blockIdx.y * 64 + lane) * V;
+    const bool live = col < hidden;
+    float wr[EMAX][V], dw[EMAX][V];
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) wr[e][i] = dw[e][i] = 0.f;
+        if (e < E && live) C::widen(*(const raw_t*)(w + (int64_t)e * hidden + col), wr[e]);
+    }
+    constexpr int U = kGateDgradTokensInFlight;
+    const int64_t stride = (int64_t)gridDim.x * 4;
+    for (int64_t t0 = (int64_t)blockIdx.x * 4 + wave; t0 < n_tokens; t0 += stride * U) {
+        raw_t a[U], xr[U];
+        float dl[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t t = t0 + u * stride;
+            dl[u] = 0.f;
+            if (t < n_tokens) {  // uniform over the wavefront
+                if (lane < E) dl[u] = to_f32<T>(d_logits[t * E + lane]);
+                if (live) {
+                    xr[u] = *(const raw_t*)(x + t * hidden + col);
+                    if (addend) a[u] = *(const raw_t*)(addend + t * hidden + col);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t t = t0 + u * stride;
+            if (t >= n_tokens || !live) break;
+            float acc[V], xv[V];
+            C::widen(xr[u], xv);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] = 0.f;
+#pragma unroll
+            for (int e = 0; e < EMAX; ++e) {
+                const float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(dl[u]), e));  // 0 for e >= E
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    acc[i] = fmaf(d, wr[e][i], acc[i]);
+                    dw[e][i] = fmaf(d, xv[i], dw[e][i]);
+                }
+            }
+            if (addend) {
+                float av[V];
+                C::widen(a[u], av);
+                C::round_all(acc);
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] += av[i];
+            }
+            *(raw_t*)(d_x + t * hidden + col) = C::narrow(acc);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+            for (int i = 0; i < V; ++i) red[wave - 1][e * V + i][lane] = dw[e][i];
+    }
+    __syncthreads();
+    if (wave == 0 && live) {
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e) {  // unrolled with a test inside: an index the compiler cannot see would move dw out of the registers
+            if (e >= E) break;
+            float* dst = partial + ((int64_t)blockIdx.x * E + e) * hidden + col;
+#pragma unroll
+            for (int i = 0; i < V; i += 4) {
+                f32x4_t o;
+                o.x = ((dw[e][i] + red[0][e * V + i][lane]) + red[1][e * V + i][lane]) + red[2][e * V + i][lane];
+                o.y = ((dw[e][i + 1] + red[0][e * V + i + 1][lane]) + red[1][e * V + i + 1][lane]) + red[2][e * V + i + 1][lane];
+                o.z = ((dw[e][i + 2] + red[0][e * V + i + 2][lane]) + red[1][e * V + i + 2][lane]) + red[2][e * V + i + 2][lane];
+                o.w = ((dw[e][i + 3] + red[0][e * V + i + 3][lane]) + red[1][e * V + i + 3][lane]) + red[2][e * V + i + 3][lane];
+                *(f32x4_t*)(dst + i) = o;
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float* __restrict__ partial, int n_partials, int64_t n,
+                                                                T* __restrict__ d_w) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    int g = 0;
+    for (; g + 16 <= n_partials; g += 16) {  // sixteen loads in flight, added in block order
+        float v[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = partial[(int64_t)(g + j) * n + i];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s += v[j];
+    }
+    for (; g < n_partials; ++g) s += partial[(int64_t)g * n + i];
+    d_w[i] = from_f32<T>(s);
+}
+
+// token groups (= partial sums of d_w) of a gate_bwd launch: about a thousand blocks over the column slabs, at least one
+// round of four tokens per block
+int gate_bwd_groups(int64_t n_tokens, int64_t hidden, int V) {
+    const int64_t slabs = (hidden + 64 * V - 1) / (64 * V);
+    int64_t g = 1024 / slabs;
+    g = g < 8 ? 8 : (g > 128 ? 128 : g);
+    const int64_t need = (n_tokens + 3) / 4;
+    if (g > need) g = need;
+    return (int)(g < 1 ? 1 : g);
+}
+
+template <typename T, int V>
+void launch_gate_bwd(hipStream_t st, const void* d_logits, const void* w, const void* addend, const void* x, int64_t n_tokens,
+                     int E, int64_t hidden, void* d_x, void* d_w, float* partial) {
+    const int groups = gate_bwd_groups(n_tokens, hidden, V);
+    const dim3 grid((unsigned)groups, (unsigned)((hidden + 64 * V - 1) / (64 * V)));
+    gate_bwd_kernel<T, V><<<grid, dim3(256), 0, st>>>((const T*)d_logits, (const T*)w, (const T*)addend, (const T*)x, n_tokens, E,
+                                                      hidden, (T*)d_x, partial);
+    const int64_t n = (int64_t)E * hidden;
+    gate_wgrad_reduce_kernel<T><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(partial, groups, n, (T*)d_w);
+}
+
 }  // namespace
 
 extern "C" int picomoe_route_partials(int64_t n_tokens, int num_experts) {
@@ -403,5 +641,48 @@ extern "C" int picomoe_balance(const int* counts, const float* colsum_partial, i
     PICOMOE_CHECK_ARG(!aux_out || (colsum_partial && n_partials >= 1));
     hipLaunchKernelGGL(balance_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, counts, colsum_partial, n_partials,
                        n_tokens, num_experts, top_k, aux_coef, bias_rate, aux_out, expert_bias);
+    return picomoe_launch_status();
+}
+
+extern "C" int64_t picomoe_gate_bwd_workspace_bytes(int dtype, int64_t n_tokens, int num_experts, int64_t hidden) {
+    if ((dtype != PICOMOE_F32 && dtype != PICOMOE_BF16) || n_tokens < 0 || num_experts < 1 || hidden < 1) return -1;
+    if (num_experts > kGateBwdMaxExperts) return 0;  // no fused weight gradient for this gate
+    return (int64_t)gate_bwd_groups(n_tokens, hidden, dtype == PICOMOE_BF16 ? 8 : 4) * num_experts * hidden * (int64_t)sizeof(float);
+}
+
+extern "C" int picomoe_gate_bwd(const void* d_logits, const void* gate_w, const void* addend, const void* tokens, int dtype,
+                                int64_t n_tokens, int num_experts, int64_t hidden, void* d_x, void* d_w, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+    PICOMOE_CHECK_ARG(dtype == PICOMOE_F32 || dtype == PICOMOE_BF16);
+    PICOMOE_CHECK_ARG(n_tokens >= 0 && hidden > 0 && num_experts >= 1);
+    PICOMOE_CHECK_ARG(num_experts <= (d_w ? kGateBwdMaxExperts : kGateDgradMaxExperts));
+    PICOMOE_CHECK_ARG(hidden % (dtype == PICOMOE_BF16 ? 8 : 4) == 0 && hidden < (1ll << 31));
+    hipStream_t st = (hipStream_t)stream;
+    if (n_tokens == 0) {
+        if (d_w) {  // the sum over no tokens: the reduction of zero partial sums writes the zeros (a kernel, so that a graph capture holds no memset node)
+            const int64_t n = (int64_t)num_experts * hidden;
+            if (dtype == PICOMOE_BF16)
+                gate_wgrad_reduce_kernel<uint16_t><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(nullptr, 0, n, (uint16_t*)d_w);
+            else
+                gate_wgrad_reduce_kernel<float><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(nullptr, 0, n, (float*)d_w);
+            return picomoe_launch_status();
+        }
+        return PICOMOE_OK;
+    }
+    PICOMOE_CHECK_ARG(d_logits && gate_w && d_x);
+    PICOMOE_CHECK_ARG((uintptr_t)gate_w % 16 == 0 && (uintptr_t)addend % 16 == 0 && (uintptr_t)d_x % 16 == 0);
+    if (!d_w) {
+        if (dtype == PICOMOE_BF16)
+            launch_gate_dgrad<uint16_t, 8>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
+        else
+            launch_gate_dgrad<float, 4>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
+        return picomoe_launch_status();
+    }
+    PICOMOE_CHECK_ARG(tokens && workspace && (uintptr_t)tokens % 16 == 0 && (uintptr_t)workspace % 16 == 0);
+    PICOMOE_CHECK_ARG(workspace_bytes >= picomoe_gate_bwd_workspace_bytes(dtype, n_tokens, num_experts, hidden));
+    if (dtype == PICOMOE_BF16)
+        launch_gate_bwd<uint16_t, 8>(st, d_logits, gate_w, addend, tokens, n_tokens, num_experts, hidden, d_x, d_w, (float*)workspace);
+    else
+        launch_gate_bwd<float, 4>(st, d_logits, gate_w, addend, tokens, n_tokens, num_experts, hidden, d_x, d_w, (float*)workspace);
     return picomoe_launch_status();
 }

@@ -160,18 +160,33 @@ class MoELayer(nn.Module):
     def forward(self, x):
         batch_size, seq_length, _ = x.shape
         tokens = x.reshape(-1, self.hidden_size)
-        topk_idx, topk_weights = self._route(tokens)
+        tokens, router_logits = self._gate(tokens)
+        topk_idx, topk_weights = self._route(tokens, router_logits)
         if self.ep_capacity_factor > 0:
             expert_out = self._moe_capped(tokens, topk_idx, topk_weights)
         else:
             expert_out = self._moe_naive(tokens, topk_idx, topk_weights)
         return expert_out.view(batch_size, seq_length, self.hidden_size)
 
-    def _route(self, tokens):
+    def _gate(self, tokens):
+        """(tokens, router logits).  With a gate the fused kernel takes (no bias, at most 16 experts, no module hooks to
+        honour) and a token gradient to carry, the tokens come back as the second output of the gate's autograd node, so that
+        their whole gradient -- through the router and through everything else that reads them -- is written by one kernel."""
+        gate = self.gate
+        fused = (gate.bias is None and torch.is_grad_enabled() and tokens.requires_grad
+                 and _ops.gate_dgrad_supported(tokens, gate.weight)
+                 and not (gate._forward_hooks or gate._forward_pre_hooks or gate._backward_hooks or gate._backward_pre_hooks))
+        if not fused:
+            return tokens, gate(tokens)
+        router_logits, tokens = _ops.gate_tap(tokens.contiguous(), gate.weight)
+        return tokens, router_logits
+
+    def _route(self, tokens, router_logits=None):
         """Router: top-k expert selection + gate weights; stashes the aux loss and steps the loss-free bias
         (training only), all inside the router kernels."""
         _lib.require_cuda(tokens)
-        router_logits = self.gate(tokens)
+        if router_logits is None:
+            router_logits = self.gate(tokens)
         balance = self.training and (self.router_aux_loss_coef > 0 or self.use_loss_free)
         # fp32 view or copy of the bias: the router kernel reads it for the selection, the balance kernel that
         # follows on the same stream steps it in place

@@ -583,3 +583,46 @@ def test_shared_expert_on_a_second_stream_changes_nothing(gpu, dtype):
         assert len(step_s) == len(step_o)
         for a, b in zip(step_s, step_o):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("n_shared", [0, 1])
+def test_fused_gate_gradient_equals_the_gate_as_a_plain_linear(gpu, dtype, rtol, n_shared):
+    """The token gradient written by one kernel (expert path + router path) against the same layer with its gate run as a
+    plain ``nn.Linear`` node (a forward hook on the gate switches the fused node off): same output and expert
+    gradients bit for bit -- the forward is the same launches -- and d x and d gate.weight within the dtype's bar; with a shared expert
+    the tokens have a third reader."""
+    cfg = make_config(hidden=256, inter=128, num_experts=8, top_k=2, n_shared=n_shared)
+    moe = build(cfg, seed=11, std=0.05, dtype=dtype)
+    moe.ep_overlap = False
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(3, 50, 256, generator=g).to(dtype)
+    up = torch.randn(3, 50, 256, generator=g).to(dtype)
+
+    def run():
+        moe.zero_grad(set_to_none=True)
+        xin = x.cuda().requires_grad_(True)
+        out = moe(xin)
+        out.backward(up.cuda())
+        return out.detach().clone(), xin.grad.clone(), {n: p.grad.clone() for n, p in moe.named_parameters()}
+
+    import picotron_amd._ops as _ops
+    calls = []
+    real = _ops.gate_tap
+    _ops.gate_tap = lambda *a: (calls.append(1), real(*a))[1]
+    try:
+        out_f, dx_f, grads_f = run()
+        assert calls == [1]
+        handle = moe.gate.register_forward_hook(lambda m, i, o: None)
+        out_p, dx_p, grads_p = run()
+        handle.remove()
+        assert calls == [1]
+    finally:
+        _ops.gate_tap = real
+    assert torch.equal(out_f, out_p)
+    for name in grads_f:
+        if name == "gate.weight":                 # d_logits.T @ x as a GEMM of the library's choosing on either side
+            assert_close(grads_f[name], grads_p[name], rtol, name)
+        else:
+            assert torch.equal(grads_f[name], grads_p[name]), name
+    assert_close(dx_f, dx_p, rtol, "d x")

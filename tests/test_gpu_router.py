@@ -121,3 +121,84 @@ def test_route_backward_matches_autograd(gpu, E, k, norm):
     _, rw2, _ = O.softmax_topk_route(lr2, k, None, norm)
     (rw2 * dw).sum().backward()
     assert (lg2.grad.cpu() - lr2.grad).abs().max().item() <= 1e-5 * lr2.grad.abs().max().item() + 1e-9
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,H", [(700, 8, 4096), (2100, 8, 264), (5, 3, 72), (1, 1, 8), (600, 16, 2048), (33, 9, 520), (0, 8, 64),
+                                   (8192, 8, 2048)])
+@pytest.mark.parametrize("with_addend", [True, False])
+@pytest.mark.parametrize("with_weight_grad", [True, False])
+def test_gate_bwd_is_the_linear_backward_plus_the_addend(gpu, dtype, T, E, H, with_addend, with_weight_grad):
+    """d_x = addend + d_logits @ W against float64 arithmetic with the kernel's two roundings (product, then sum) and
+    d_W = d_logits.T @ x against float64 rounded once: fp32 within 1e-5 of the largest element, bf16 within 1e-2 (one
+    rounding step of either).  Token counts above and below the grid, more than four tokens per wavefront, widths that
+    leave lanes without columns, 1..16 experts (the weight gradient is fused up to 8; above, None comes back)."""
+    from picotron_amd import _ops
+
+    g = torch.Generator().manual_seed(T * 31 + E * 7 + H)
+    d_logits = torch.randn(T, E, generator=g).to(dtype)
+    w = torch.randn(E, H, generator=g).to(dtype)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    addend = (3 * torch.randn(T, H, generator=g)).to(dtype) if with_addend else None
+    d_x, d_w = _ops.gate_bwd(d_logits.cuda(), w.cuda(), addend.cuda() if with_addend else None, x.cuda(), with_weight_grad)
+    torch.cuda.synchronize()
+    ref = (d_logits.double() @ w.double()).to(dtype).double()
+    if with_addend:
+        ref = (ref + addend.double()).to(dtype).double()
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    got = d_x.cpu().double()
+    assert got.shape == (T, H) and torch.isfinite(got).all()
+    if T:
+        assert (got - ref).abs().max() <= tol * ref.abs().amax()
+    assert (d_w is not None) == (with_weight_grad and E <= 8)
+    if d_w is not None:
+        ref_w = (d_logits.double().t() @ x.double()).to(dtype).double()
+        got_w = d_w.cpu().double()
+        assert got_w.shape == (E, H) and torch.isfinite(got_w).all()
+        assert (got_w - ref_w).abs().max() <= tol * max(float(ref_w.abs().amax()), 1e-30)
+        if T == 0:
+            assert not got_w.any()
+
+
+def test_gate_weight_gradient_has_one_fixed_summation_order(gpu):
+    """Two launches on the same inputs give the same bits (block sums are added in block order, no atomics)."""
+    from picotron_amd import _ops
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    T, E, H = 5000, 8, 1024
+    dl = torch.randn(T, E, generator=g, device="cuda").bfloat16()
+    w = torch.randn(E, H, generator=g, device="cuda").bfloat16()
+    x = torch.randn(T, H, generator=g, device="cuda").bfloat16()
+    a = _ops.gate_bwd(dl, w, None, x, True)
+    b = _ops.gate_bwd(dl, w, None, x, True)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_gate_tap_gradients_equal_the_linear_beside_its_readers(gpu):
+    """The autograd node that hands the tokens through gives the gradients of `linear(x, W)` with a second reader of x:
+    d x and d W against float64 autograd of the same graph (fp32: 1e-5 of the largest element)."""
+    from picotron_amd import _ops
+
+    g = torch.Generator().manual_seed(5)
+    T, E, H = 300, 8, 512
+    x = torch.randn(T, H, generator=g)
+    w = 0.1 * torch.randn(E, H, generator=g)
+    m = torch.randn(T, H, generator=g)
+    c = torch.randn(T, E, generator=g)
+    xd, wd = x.cuda().requires_grad_(), w.cuda().requires_grad_()
+    assert _ops.gate_dgrad_supported(xd, wd)
+    logits, tap = _ops.gate_tap(xd, wd)
+    ((logits * c.cuda()).sum() + (tap * m.cuda()).sum()).backward()
+    x64, w64 = x.double().requires_grad_(), w.double().requires_grad_()
+    ((torch.nn.functional.linear(x64, w64) * c.double()).sum() + (x64 * m.double()).sum()).backward()
+    for got, ref in ((xd.grad, x64.grad), (wd.grad, w64.grad)):
+        assert (got.cpu().double() - ref).abs().max() <= 1e-5 * ref.abs().max()
+    # only the logits read: the gradient is the plain product; only the tokens read: it is handed through
+    xd.grad = None
+    logits, tap = _ops.gate_tap(xd, wd)
+    (logits * c.cuda()).sum().backward()
+    assert (xd.grad.cpu().double() - c.double() @ w.double()).abs().max() <= 1e-5 * 10
+    xd.grad = None
+    logits, tap = _ops.gate_tap(xd, wd)
+    (tap * m.cuda()).sum().backward()
+    assert torch.equal(xd.grad.cpu(), m)

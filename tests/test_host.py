@@ -61,8 +61,19 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.picomoe_dispatch_fp8(null, 1, 0, 64, null, 2, 0, null, null, null, null, null, null) == 0   # no tokens
     assert lib.picomoe_dispatch_fp8(null, 1, 4, 64, null, 17, 8, null, null, null, null, null, null) == 1  # top_k > 16
     assert lib.picomoe_dispatch_fp8(null, 1, 4, 64, null, 2, 8, null, counts, null, null, null, null) == 1 # codes without scales
+    a16 = ctypes.c_void_p(64)
+    assert lib.picomoe_gate_bwd(null, null, null, null, 1, 0, 8, 4096, null, null, null, 0, null) == 0            # no tokens, no d_w
+    assert lib.picomoe_gate_bwd(a16, a16, null, null, 1, 4, 17, 4096, a16, null, null, 0, null) == 1             # more than 16 experts
+    assert lib.picomoe_gate_bwd(a16, a16, null, a16, 1, 4, 9, 4096, a16, a16, a16, 1 << 30, null) == 1           # d_w with more than 8
+    assert lib.picomoe_gate_bwd(a16, a16, null, null, 1, 4, 8, 4100, a16, null, null, 0, null) == 1              # row not in 16-byte chunks
+    assert lib.picomoe_gate_bwd(a16, a16, ctypes.c_void_p(72), null, 0, 4, 8, 64, a16, null, null, 0, null) == 1 # misaligned addend
+    assert lib.picomoe_gate_bwd(a16, a16, null, a16, 1, 4, 8, 4096, a16, a16, a16, 16, null) == 1                # workspace too small
+    assert lib.picomoe_gate_bwd_workspace_bytes(1, 8192, 8, 4096) == 128 * 8 * 4096 * 4
+    assert lib.picomoe_gate_bwd_workspace_bytes(0, 10, 4, 64) == 3 * 4 * 64 * 4          # three groups of four tokens
+    assert lib.picomoe_gate_bwd_workspace_bytes(1, 8192, 9, 4096) == 0 and lib.picomoe_gate_bwd_workspace_bytes(2, 1, 1, 1) == -1
     assert lib.picomoe_ffn_kernel_family(1, 4096, 14336) == 1 and lib.picomoe_ffn_kernel_family(0, 256, 512) == 2
     assert lib.picomoe_ffn_kernel_family(1, 100, 36) == 0 and lib.picomoe_ffn_kernel_family(0, 16, 32) == 0
+    assert b"fixed scratch" in lib.picomoe_error_string(2) and b"tile numbering" in lib.picomoe_error_string(2)
     with pytest.raises(_lib.PicomoeError):
         _lib.check(1, "demo")
 

@@ -85,7 +85,7 @@ def test_static_plan_refuses_what_does_not_fit(gpu):
     assert lib.picomoe_permute_workspace_bytes(R, E) > lib.picomoe_permute_plan_static_max_bytes()
     idx = torch.zeros(R, dtype=torch.int64, device=gpu)
     rc, _ = _plan(lib, _lib, idx, E, 0, 0, static=True)
-    assert rc == 2 and b"larger than the fixed scratch" in lib.picomoe_error_string(rc)
+    assert rc == 2 and b"exceeds the fixed scratch" in lib.picomoe_error_string(rc)
     with pytest.raises(_lib.PicomoeError):
         _lib.check(rc, "picomoe_permute_plan_static")
     # the largest plan that fits: 255 blocks x 1024 experts
