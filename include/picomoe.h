@@ -92,11 +92,11 @@ int picomoe_balance(const int* counts, const float* colsum_partial, int n_partia
 /* Backward of the router's gate Linear, EP/expert_parallel.py:65 and :174 (`self.gate = nn.Linear(hidden, num_experts,
  * bias=False)`, `router_logits = self.gate(tokens)`: autograd's d_tokens = d_logits @ gate.weight and d_weight =
  * d_logits.T @ tokens), together with autograd's sum of the tokens' gradient paths (through the router and through the
- * experts), in one pass over the tokens: d_x[t] = addend[t] + d_logits[t] @ gate_w and, when d_w is given,
+ * experts), in one read of each operand: d_x[t] = addend[t] + d_logits[t] @ gate_w and, when d_w is given,
  * d_w[e] = sum_t d_logits[t, e] * tokens[t] (fp32 sums in a fixed order, rounded once).  d_logits [n_tokens, num_experts],
  * gate_w and d_w [num_experts, hidden], addend (NULL = zeros), tokens and d_x [n_tokens, hidden], all in dtype; the product
  * d_logits @ gate_w is rounded to dtype before the sum with the addend, as a GEMM followed by an add rounds.
- * num_experts <= 16 for d_x alone (tokens, d_w, workspace NULL) and <= 8 with d_w, which needs `workspace` of
+ * Either output may be NULL.  num_experts <= 16 for d_x alone (tokens, d_w, workspace NULL) and <= 8 with d_w, which needs `workspace` of
  * picomoe_gate_bwd_workspace_bytes(...) bytes (0 = this gate has no fused weight gradient; -1 = bad arguments); hidden a
  * multiple of 16 bytes, pointers 16-byte aligned: PICOMOE_ERR_ARG otherwise (a caller keeps the library GEMMs for wider
  * routers). */

@@ -95,7 +95,7 @@ def gate_dgrad_supported(tokens, weight):
 
 def gate_bwd(d_logits, weight, addend, tokens, want_weight_grad):
     """(d_tokens, d_weight or None) of ``linear(tokens, weight)`` with ``addend`` (the tokens' gradient from their other
-    readers, or None) summed in: one pass over the tokens.  d_weight is None when it was not asked for or the kernel has no
+    readers, or None) summed in.  d_weight is None when it was not asked for or the kernel has no
     fused form for this many experts (the caller then runs the GEMM)."""
     lib = _lib.load()
     T, H = tokens.shape
@@ -123,8 +123,8 @@ class _GateTap(torch.autograd.Function):
     """(logits, tokens) = (tokens @ weight.T, tokens): the router's gate Linear with the tokens handed through.
 
     Everything else that reads the tokens (dispatch, shared expert) reads the second output, so autograd delivers the sum
-    of their gradients here together with d_logits, and one kernel writes d_tokens = that sum + d_logits @ weight and, for
-    up to 8 experts, d_weight = d_logits.T @ tokens -- where an ``nn.Linear`` node beside the others costs a GEMM that
+    of their gradients here together with d_logits, and one kernel writes d_tokens = that sum + d_logits @ weight (for up
+    to 8 experts a second one sums d_weight = d_logits.T @ tokens from one read of the tokens) -- where an ``nn.Linear`` node beside the others costs a GEMM that
     writes [T, H], an add that reads two and writes one, and a GEMM with an E-row output that reads the tokens at a
     fraction of the memory rate.  The logits stay a library GEMM, as in the reference (expert_parallel.py:65, :174).
     """

@@ -445,17 +445,18 @@ void launch_gate_dgrad(hipStream_t st, const void* d_logits, const void* w, cons
                                                                                   (const T*)addend, n_tokens, E, hidden, (T*)out);
 }
 
-// The same pass with the gate's weight gradient beside it: d_w[e, :] = sum_t d_logits[t, e] * x[t, :] is E more
-// multiply-adds per element of x read, against columns the thread already owns, so reading x here (one more stream)
-// replaces a GEMM with an 8-row output that runs at a fifth of the memory rate.  A block's four wavefronts own the same
-// 64 * V columns and every fourth token of the block's share; their sums meet in LDS in wave order, the blocks' sums in
-// `partial` [gridDim.x][E][hidden] fp32, which gate_wgrad_reduce_kernel adds in block order: no atomics, one fixed order.
+// The gate's weight gradient d_w[e, :] = sum_t d_logits[t, e] * x[t, :]: E multiply-adds per element of x read, against
+// columns the thread owns, so it runs at the rate x can be read -- a GEMM with an E-row output reaches a fifth of that.
+// A block's four wavefronts own the same 64 * V columns and every fourth token of the block's share; their sums meet in
+// LDS in wave order, the blocks' sums in `partial` [gridDim.x][E][hidden] fp32, which gate_wgrad_reduce_kernel adds in
+// block order: no atomics, one fixed order.  (One kernel for d_x and d_w together was measured and dropped: with W and
+// the sums both in registers two wavefronts fit a SIMD and the pass ran at 2.8 TB/s, no faster than the two apart.)
 constexpr int kGateBwdMaxExperts = 8;
+constexpr int kGateWgradTokensInFlight = 4;  // per batch, two batches
 
 template <typename T, int V>
-__global__ __launch_bounds__(256) void gate_bwd_kernel(const T* __restrict__ d_logits, const T* __restrict__ w,
-                                                       const T* __restrict__ addend, const T* __restrict__ x, int64_t n_tokens,
-                                                       int E, int64_t hidden, T* __restrict__ d_x, float* __restrict__ partial) {
+__global__ __launch_bounds__(256) void gate_wgrad_kernel(const T* __restrict__ d_logits, const T* __restrict__ x, int64_t n_tokens,
+                                                         int E, int64_t hidden, float* __restrict__ partial) {
     typedef Cols<T, V> C;
     typedef typename C::raw_t raw_t;
     constexpr int EMAX = kGateBwdMaxExperts;
@@ -463,56 +464,51 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const T* __restrict__ d_l
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t col = ((int64_t)blockIdx.y * 64 + lane) * V;
     const bool live = col < hidden;
-    float wr[EMAX][V], dw[EMAX][V];
+    float dw[EMAX][V];
 #pragma unroll
-    for (int e = 0; e < EMAX; ++e) {
+    for (int e = 0; e < EMAX; ++e)
 #pragma unroll
-        for (int i = 0; i < V; ++i) wr[e][i] = dw[e][i] = 0.f;
-        if (e < E && live) C::widen(*(const raw_t*)(w + (int64_t)e * hidden + col), wr[e]);
-    }
-    constexpr int U = kGateDgradTokensInFlight;
-    const int64_t stride = (int64_t)gridDim.x * 4;
-    for (int64_t t0 = (int64_t)blockIdx.x * 4 + wave; t0 < n_tokens; t0 += stride * U) {
-        raw_t a[U], xr[U];
-        float dl[U];
+        for (int i = 0; i < V; ++i) dw[e][i] = 0.f;
+    // two batches of U tokens: the loads of one are in flight while the other is summed
+    constexpr int U = kGateWgradTokensInFlight;
+    const int64_t stride = (int64_t)gridDim.x * 4, step = stride * U;
+    auto load = [&](raw_t (&xr)[U], float (&dl)[U], int64_t t0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int64_t t = t0 + u * stride;
             dl[u] = 0.f;
             if (t < n_tokens) {  // uniform over the wavefront
                 if (lane < E) dl[u] = to_f32<T>(d_logits[t * E + lane]);
-                if (live) {
-                    xr[u] = *(const raw_t*)(x + t * hidden + col);
-                    if (addend) a[u] = *(const raw_t*)(addend + t * hidden + col);
-                }
+                if (live) xr[u] = *(const raw_t*)(x + t * hidden + col);
             }
         }
+    };
+    auto accumulate = [&](const raw_t (&xr)[U], const float (&dl)[U], int64_t t0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t t = t0 + u * stride;
-            if (t >= n_tokens || !live) break;
-            float acc[V], xv[V];
+            if (t0 + u * stride >= n_tokens || !live) break;
+            float xv[V];
             C::widen(xr[u], xv);
-#pragma unroll
-            for (int i = 0; i < V; ++i) acc[i] = 0.f;
 #pragma unroll
             for (int e = 0; e < EMAX; ++e) {
                 const float d = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(dl[u]), e));  // 0 for e >= E
 #pragma unroll
-                for (int i = 0; i < V; ++i) {
-                    acc[i] = fmaf(d, wr[e][i], acc[i]);
-                    dw[e][i] = fmaf(d, xv[i], dw[e][i]);
-                }
+                for (int i = 0; i < V; ++i) dw[e][i] = fmaf(d, xv[i], dw[e][i]);
             }
-            if (addend) {
-                float av[V];
-                C::widen(a[u], av);
-                C::round_all(acc);
-#pragma unroll
-                for (int i = 0; i < V; ++i) acc[i] += av[i];
-            }
-            *(raw_t*)(d_x + t * hidden + col) = C::narrow(acc);
         }
+    };
+    raw_t xa[U], xb[U];
+    float da[U], db[U];
+    int64_t t0 = (int64_t)blockIdx.x * 4 + wave;
+    if (t0 < n_tokens) load(xa, da, t0);
+    while (t0 < n_tokens) {
+        if (t0 + step < n_tokens) load(xb, db, t0 + step);
+        accumulate(xa, da, t0);
+        t0 += step;
+        if (t0 >= n_tokens) break;
+        if (t0 + step < n_tokens) load(xa, da, t0 + step);
+        accumulate(xb, db, t0);
+        t0 += step;
     }
     if (wave > 0) {
 #pragma unroll
@@ -557,24 +553,23 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float* __r
     d_w[i] = from_f32<T>(s);
 }
 
-// token groups (= partial sums of d_w) of a gate_bwd launch: about a thousand blocks over the column slabs, at least one
-// round of four tokens per block
+// token groups (= partial sums of d_w) of a weight-gradient launch: three blocks per CU over the column slabs (what the
+// 48 KB of LDS a block takes allows), at least one round of four tokens per block
 int gate_bwd_groups(int64_t n_tokens, int64_t hidden, int V) {
     const int64_t slabs = (hidden + 64 * V - 1) / (64 * V);
-    int64_t g = 1024 / slabs;
-    g = g < 8 ? 8 : (g > 128 ? 128 : g);
+    int64_t g = 768 / slabs;
+    g = g < 8 ? 8 : (g > 96 ? 96 : g);
     const int64_t need = (n_tokens + 3) / 4;
     if (g > need) g = need;
     return (int)(g < 1 ? 1 : g);
 }
 
 template <typename T, int V>
-void launch_gate_bwd(hipStream_t st, const void* d_logits, const void* w, const void* addend, const void* x, int64_t n_tokens,
-                     int E, int64_t hidden, void* d_x, void* d_w, float* partial) {
+void launch_gate_wgrad(hipStream_t st, const void* d_logits, const void* x, int64_t n_tokens, int E, int64_t hidden, void* d_w,
+                       float* partial) {
     const int groups = gate_bwd_groups(n_tokens, hidden, V);
     const dim3 grid((unsigned)groups, (unsigned)((hidden + 64 * V - 1) / (64 * V)));
-    gate_bwd_kernel<T, V><<<grid, dim3(256), 0, st>>>((const T*)d_logits, (const T*)w, (const T*)addend, (const T*)x, n_tokens, E,
-                                                      hidden, (T*)d_x, partial);
+    gate_wgrad_kernel<T, V><<<grid, dim3(256), 0, st>>>((const T*)d_logits, (const T*)x, n_tokens, E, hidden, partial);
     const int64_t n = (int64_t)E * hidden;
     gate_wgrad_reduce_kernel<T><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(partial, groups, n, (T*)d_w);
 }
@@ -669,20 +664,16 @@ extern "C" int picomoe_gate_bwd(const void* d_logits, const void* gate_w, const 
         }
         return PICOMOE_OK;
     }
-    PICOMOE_CHECK_ARG(d_logits && gate_w && d_x);
-    PICOMOE_CHECK_ARG((uintptr_t)gate_w % 16 == 0 && (uintptr_t)addend % 16 == 0 && (uintptr_t)d_x % 16 == 0);
-    if (!d_w) {
-        if (dtype == PICOMOE_BF16)
-            launch_gate_dgrad<uint16_t, 8>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
-        else
-            launch_gate_dgrad<float, 4>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
-        return picomoe_launch_status();
+    PICOMOE_CHECK_ARG(d_logits && (d_x || d_w));
+    if (d_x) PICOMOE_CHECK_ARG(gate_w && (uintptr_t)gate_w % 16 == 0 && (uintptr_t)addend % 16 == 0 && (uintptr_t)d_x % 16 == 0);
+    if (d_w) {
+        PICOMOE_CHECK_ARG(tokens && workspace && (uintptr_t)tokens % 16 == 0 && (uintptr_t)workspace % 16 == 0);
+        PICOMOE_CHECK_ARG(workspace_bytes >= picomoe_gate_bwd_workspace_bytes(dtype, n_tokens, num_experts, hidden));
     }
-    PICOMOE_CHECK_ARG(tokens && workspace && (uintptr_t)tokens % 16 == 0 && (uintptr_t)workspace % 16 == 0);
-    PICOMOE_CHECK_ARG(workspace_bytes >= picomoe_gate_bwd_workspace_bytes(dtype, n_tokens, num_experts, hidden));
-    if (dtype == PICOMOE_BF16)
-        launch_gate_bwd<uint16_t, 8>(st, d_logits, gate_w, addend, tokens, n_tokens, num_experts, hidden, d_x, d_w, (float*)workspace);
-    else
-        launch_gate_bwd<float, 4>(st, d_logits, gate_w, addend, tokens, n_tokens, num_experts, hidden, d_x, d_w, (float*)workspace);
+    const bool bf16 = dtype == PICOMOE_BF16;
+    if (d_x && bf16) launch_gate_dgrad<uint16_t, 8>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
+    if (d_x && !bf16) launch_gate_dgrad<float, 4>(st, d_logits, gate_w, addend, n_tokens, num_experts, hidden, d_x);
+    if (d_w && bf16) launch_gate_wgrad<uint16_t, 8>(st, d_logits, tokens, n_tokens, num_experts, hidden, d_w, (float*)workspace);
+    if (d_w && !bf16) launch_gate_wgrad<float, 4>(st, d_logits, tokens, n_tokens, num_experts, hidden, d_w, (float*)workspace);
     return picomoe_launch_status();
 }

@@ -68,7 +68,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.picomoe_gate_bwd(a16, a16, null, null, 1, 4, 8, 4100, a16, null, null, 0, null) == 1              # row not in 16-byte chunks
     assert lib.picomoe_gate_bwd(a16, a16, ctypes.c_void_p(72), null, 0, 4, 8, 64, a16, null, null, 0, null) == 1 # misaligned addend
     assert lib.picomoe_gate_bwd(a16, a16, null, a16, 1, 4, 8, 4096, a16, a16, a16, 16, null) == 1                # workspace too small
-    assert lib.picomoe_gate_bwd_workspace_bytes(1, 8192, 8, 4096) == 128 * 8 * 4096 * 4
+    assert lib.picomoe_gate_bwd_workspace_bytes(1, 8192, 8, 4096) == 96 * 8 * 4096 * 4
     assert lib.picomoe_gate_bwd_workspace_bytes(0, 10, 4, 64) == 3 * 4 * 64 * 4          # three groups of four tokens
     assert lib.picomoe_gate_bwd_workspace_bytes(1, 8192, 9, 4096) == 0 and lib.picomoe_gate_bwd_workspace_bytes(2, 1, 1, 1) == -1
     assert lib.picomoe_ffn_kernel_family(1, 4096, 14336) == 1 and lib.picomoe_ffn_kernel_family(0, 256, 512) == 2
