@@ -98,7 +98,7 @@ int picomoe_balance(const int* counts, const float* colsum_partial, int n_partia
  * d_logits @ gate_w is rounded to dtype before the sum with the addend, as a GEMM followed by an add rounds.
  * Either output may be NULL.  num_experts <= 16 for d_x alone (tokens, d_w, workspace NULL) and <= 8 with d_w, which needs `workspace` of
  * picomoe_gate_bwd_workspace_bytes(...) bytes (0 = this gate has no fused weight gradient; -1 = bad arguments); hidden a
- * multiple of 16 bytes, pointers 16-byte aligned: PICOMOE_ERR_ARG otherwise (a caller keeps the library GEMMs for wider
+ * multiple of 16 bytes and at most 2^22, pointers 16-byte aligned: PICOMOE_ERR_ARG otherwise (a caller keeps the library GEMMs for wider
  * routers). */
 int64_t picomoe_gate_bwd_workspace_bytes(int dtype, int64_t n_tokens, int num_experts, int64_t hidden);
 int picomoe_gate_bwd(const void* d_logits, const void* gate_w, const void* addend, const void* tokens, int dtype,

@@ -90,7 +90,8 @@ def gate_dgrad_supported(tokens, weight):
     """Whether picomoe_gate_bwd takes this gate: up to 16 experts, fp32 or bf16 in one dtype, rows of whole 16-byte chunks."""
     return (tokens.is_cuda and tokens.dim() == 2 and weight.dim() == 2 and tokens.dtype == weight.dtype
             and tokens.dtype in (torch.float32, torch.bfloat16) and weight.shape[0] <= GATE_DGRAD_MAX_EXPERTS
-            and (tokens.shape[1] * tokens.element_size()) % 16 == 0 and not torch.is_autocast_enabled())
+            and (tokens.shape[1] * tokens.element_size()) % 16 == 0 and tokens.shape[1] <= 1 << 22
+            and not torch.is_autocast_enabled())
 
 
 def gate_bwd(d_logits, weight, addend, tokens, want_weight_grad):

@@ -651,7 +651,7 @@ extern "C" int picomoe_gate_bwd(const void* d_logits, const void* gate_w, const 
     PICOMOE_CHECK_ARG(dtype == PICOMOE_F32 || dtype == PICOMOE_BF16);
     PICOMOE_CHECK_ARG(n_tokens >= 0 && hidden > 0 && num_experts >= 1);
     PICOMOE_CHECK_ARG(num_experts <= (d_w ? kGateBwdMaxExperts : kGateDgradMaxExperts));
-    PICOMOE_CHECK_ARG(hidden % (dtype == PICOMOE_BF16 ? 8 : 4) == 0 && hidden < (1ll << 31));
+    PICOMOE_CHECK_ARG(hidden % (dtype == PICOMOE_BF16 ? 8 : 4) == 0 && hidden <= (1ll << 22));  // column slabs are the grid's y dimension
     hipStream_t st = (hipStream_t)stream;
     if (n_tokens == 0) {
         if (d_w) {  // the sum over no tokens: the reduction of zero partial sums writes the zeros (a kernel, so that a graph capture holds no memset node)
