@@ -764,6 +764,8 @@ def main():
             "traffic_source": measured_traffic(args.workload)[1],
             "kernel": "ffn_mfma_kernel (grouped SwiGLU GEMMs: %s)" % ", ".join(kt),
             "flop_per_step": total_flop, "gemm_ms_per_step": total_ms, "sum_of_launch_ms_per_step": sum_ms,
+            # router, plan, dispatch, combine and their backward passes: what a step spends with no grouped GEMM running
+            "step_minus_gemm_ms": result["ms_per_step"] - total_ms,
             "launches": {k: {"ms": t, "tflops": f / t / 1e9} for k, (t, f) in kt.items()},
         }
         log(f"[bench] grouped GEMM: {achieved:.0f} TFLOP/s over {total_ms:.2f} ms/step "
