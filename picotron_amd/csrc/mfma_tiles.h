@@ -132,8 +132,17 @@ __device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, i
     bool want_light;
     uint32_t L;
     if (tile_slot < g.heavy_per_xcd) {
+        // Runs of kCusPerXcd heavy tiles are dealt to the XCDs in turn (run r to XCD r mod 8) while whole deals of eight runs
+        // last, and what is left is split evenly, a contiguous eighth per XCD: every XCD still runs heavy_per_xcd tiles, but at
+        // any time the eight of them work through neighbouring column ranges of the same expert, whose rows (the A operand,
+        // re-read by every column range) then stay in the last-level cache -- with one expert per XCD the rows of eight
+        // experts pass through it at once.
         want_light = false;
-        L = xcd * g.heavy_per_xcd + tile_slot;
+        const uint32_t deals = g.heavy_per_xcd / (uint32_t)kCusPerXcd, dealt = deals * (uint32_t)kCusPerXcd;
+        if (tile_slot < dealt)
+            L = ((tile_slot / (uint32_t)kCusPerXcd) * (uint32_t)kNumXcd + xcd) * (uint32_t)kCusPerXcd + tile_slot % (uint32_t)kCusPerXcd;
+        else
+            L = dealt * (uint32_t)kNumXcd + xcd * (g.heavy_per_xcd - dealt) + (tile_slot - dealt);
         if (L >= g.heavy) return false;
     } else if (tile_slot < g.per_xcd) {
         want_light = true;
