@@ -149,11 +149,14 @@ def test_explicit_dgrad_wgrad_api(gpu, dtype):
 
 
 @pytest.mark.parametrize("H,I,counts", [(256, 512, [130, 128, 126, 0, 1, 64, 63, 0]), (100, 36, [7, 300]), (256, 384, [300, 0, 5, 257]), (512, 128, [1, 1000, 70]),
-                                        (320, 192, [300, 0, 5, 257]), (128, 448, [129, 64, 1]), (704, 320, [33, 520, 0, 256]), (192, 128, [257, 3])])
+                                        (320, 192, [300, 0, 5, 257]), (128, 448, [129, 64, 1]), (704, 320, [33, 520, 0, 256]), (192, 128, [257, 3]),
+                                        (512, 4096, [700, 3, 0, 129, 260, 515, 40, 1, 300, 256, 90, 130, 64, 257, 511, 33, 128, 127, 5, 600])])
 def test_bf16_ragged_against_oracle(gpu, H, I, counts):
     """bf16: outputs and gradients within rtol 1e-2 of the oracle (measured against the magnitude of each tensor).
-    The last four shapes are widths the 256-column tiles do not divide (hidden 320, 128, 704, 192; FFN 192, 448, 320): the
-    MFMA kernels run them with clamped loads and masked stores in the last tile column."""
+    Shapes five to eight are widths the 256-column tiles do not divide (hidden 320, 128, 704, 192; FFN 192, 448, 320): the
+    MFMA kernels run them with clamped loads and masked stores in the last tile column.  The last one has enough tiles (twenty
+    skewed experts, FFN 4096) for the tile walk to deal whole runs of 32 to the eight XCDs and still have tiles left over, in the
+    row-grouped kernels (480 heavy tiles for gate/up) and in the weight gradients (640 and 1280 tiles)."""
     from picotron_amd.expert_parallel import megakernel
 
     E = len(counts)
