@@ -166,8 +166,15 @@ __device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, i
             const uint32_t me_e = (uint32_t)uniform_i32(__shfl(me, src, 64));
             const uint32_t Le = L - tiles_before - (uint32_t)uniform_i32(__shfl(te_incl, src, 64) - __shfl(te, src, 64));
             const uint32_t start = rows_before + (uint32_t)uniform_i32(__shfl(rows_incl, src, 64)) - c_e;
-            const uint32_t nt = Le / me_e;
-            const uint32_t m = want_light ? c_e / BM : Le - nt * me_e;
+            // The expert's heavy tiles in groups of 8 tile rows: a group's tiles column by column, tile row fastest, then the
+            // next group.  32 consecutive tiles -- what an XCD's CUs run at a time -- are then an 8 x 4 patch (8 + 4 operand
+            // slices per k-step from the L2) however many rows the expert has; with all its tile rows in one column-major sweep
+            // an expert of 64 tile rows (a shared expert over 16384 tokens) gave an XCD 32 x 1 patches, 33 slices per k-step.
+            constexpr uint32_t GM = 8;
+            const uint32_t grp = Le / (GM * (uint32_t)n_tiles), in_grp = Le - grp * (GM * (uint32_t)n_tiles);
+            const uint32_t hm = want_light ? 1u : (me_e - grp * GM < GM ? me_e - grp * GM : GM);  // tile rows of this group
+            const uint32_t nt = in_grp / hm, rm = in_grp - nt * hm;
+            const uint32_t m = want_light ? c_e / BM : grp * GM + rm;
             tc->e = base + src;
             tc->m_tile = (int)m;
             tc->n_tile = (int)nt;
@@ -176,8 +183,8 @@ __device__ __forceinline__ bool locate_tile_slot(const int64_t* counts, int E, i
             tc->rows = (int)(left < (uint32_t)BM ? left : (uint32_t)BM);
             tc->a_sn = n_tiles < 4 ? n_tiles : 4;
             tc->a_si = tc->n_tile % tc->a_sn;
-            tc->b_sn = (int)(me_e < 8 ? me_e : 8);
-            tc->b_si = (int)(m % (uint32_t)tc->b_sn);
+            tc->b_sn = (int)hm;
+            tc->b_si = (int)rm;
             return true;
         }
         tiles_before += te_total;
