@@ -37,7 +37,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # A counter run cannot happen inside a timed run, so the figure is carried here together with the digest of the kernel
 # sources it was measured on: `traffic` is reported only while the sources are still those, otherwise it is null.
 MEASURED_TRAFFIC = {
-    "c5": {"bytes": 35.3e9, "algorithmic_bytes": 15.5e9, "sources": "e249dd43310dd377",
+    "c5": {"bytes": 35.3e9, "algorithmic_bytes": 15.5e9, "sources": "6a7e161c91880ec2",
            "files": ("ffn_mfma.hip", "mfma_tiles.h", "ffn.h", "common.h"),
            "summary": "profiles/ffn_mfma_kernel_mixtral_hbm_traffic.txt"},
     "c2": {"bytes": 201.6e6, "algorithmic_bytes": 201.4e6, "sources": "567861dc6e2a9e36",

@@ -161,10 +161,9 @@ __global__ __launch_bounds__(NW * 64, 1) void ffn_mfma_kernel(MfmaParams p) {
     const int l15 = lane & 15, g4 = lane >> 4;
     // k-tiles of this block: all of K, or this piece's share of it
     const int n_kt_all = MODE == kWgrad ? (int)((uint32_t)(tc.rows + BK - 1) / BK) : (int)((uint64_t)p.K / BK);
-    // (pieces is 1, 2 or 4: the quotient is a shift)
-    const int pieces_lg = tc.pieces >> 1;
-    const int kt_first = kCanSplit ? (tc.piece * n_kt_all) >> pieces_lg : 0;
-    const int n_kt = kCanSplit ? (((tc.piece + 1) * n_kt_all) >> pieces_lg) - kt_first : n_kt_all;
+    // (pieces is 1 .. 4; two 32-bit divisions per block)
+    const int kt_first = kCanSplit ? (int)((uint32_t)(tc.piece * n_kt_all) / (uint32_t)tc.pieces) : 0;
+    const int n_kt = kCanSplit ? (int)((uint32_t)((tc.piece + 1) * n_kt_all) / (uint32_t)tc.pieces) - kt_first : n_kt_all;
     // a wavefront whose 128 rows all lie past the end of the expert's segment keeps loading and synchronising
     // but skips its fragment reads and MFMAs
     // 32-row blocks of this wave's 128 rows that hold rows of the expert's segment (wgrad: all four; its ragged dimension is K)

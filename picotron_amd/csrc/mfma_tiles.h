@@ -112,10 +112,11 @@ __device__ __forceinline__ GroupedLayout grouped_layout(const int64_t* counts, i
     g.rem = 0;
     g.pieces = 1;
     if (max_pieces > 1) {
-        static_assert(kCusPerXcd == 32 && kMaxSplit == 4, "the piece count below is kCusPerXcd / rem, capped at 4, 3 -> 2");
+        static_assert(kCusPerXcd == 32 && kMaxSplit == 4, "the piece count below is kCusPerXcd / rem, capped at 4");
         const int rem = (int)(g.per_xcd % (uint32_t)kCusPerXcd);
-        int pieces = rem == 0 ? 1 : (rem <= 8 ? 4 : (rem <= 16 ? 2 : 1));
-        if (pieces > max_pieces) pieces = max_pieces == 3 ? 2 : max_pieces;
+        // as many pieces as keep rem * pieces within the XCD's 32 CUs: 4 up to 8 left-over tiles, 3 for 9 or 10, 2 up to 16
+        int pieces = rem == 0 ? 1 : (rem <= 8 ? 4 : (rem <= 10 ? 3 : (rem <= 16 ? 2 : 1)));
+        if (pieces > max_pieces) pieces = max_pieces;
         if (pieces > 1) {
             g.full = g.per_xcd - (uint32_t)rem;
             g.rem = rem;
@@ -204,9 +205,9 @@ __device__ __forceinline__ bool locate_m_grouped(const int64_t* counts, int E, i
     if (slot >= g.full && g.pieces > 1) {
         const uint32_t idx = slot - g.full;
         if (idx >= (uint32_t)(g.rem * g.pieces)) return false;
-        const int lg = g.pieces >> 1;  // pieces is 2 or 4
-        tile_slot = g.full + (idx >> lg);
-        tc->piece = (int)(idx & (uint32_t)(g.pieces - 1));
+        const uint32_t tile = idx / (uint32_t)g.pieces;  // pieces is 2, 3 or 4
+        tile_slot = g.full + tile;
+        tc->piece = (int)(idx - tile * (uint32_t)g.pieces);
         tc->pieces = g.pieces;
         tc->ws_slot = (int)((blockIdx.x % kNumXcd) * kCusPerXcd + idx);
     }
